@@ -1,0 +1,73 @@
+"""Thin Python handle on the C++ BERT driver (csrc/bert_driver.cpp) for tests
+and benchmarks: uploads seeded weights, runs the lowered encoder's call list
+eagerly or as a replayed HIP graph, fetches the output."""
+import ctypes
+
+import numpy as np
+
+from . import hom_runtime as rt
+
+
+class BertEncoder:
+    def __init__(self, layers, hidden, heads, ffn, bs, seq, vocab, gemm_mode=1, gelu_form="erf"):
+        self.drv = rt.load_driver()
+        self.dims = dict(layers=layers, hidden=hidden, heads=heads, ffn=ffn, bs=bs, seq=seq, vocab=vocab)
+        self.gemm_mode = gemm_mode
+        self.h = self.drv.homBertCreate(layers, hidden, heads, ffn, bs, seq, vocab, gemm_mode,
+                                        1 if gelu_form == "tanh" else 0)
+        assert self.h, "homBertCreate failed"
+
+    def close(self):
+        if self.h:
+            self.drv.homBertDestroy(self.h)
+            self.h = None
+
+    def _upload(self, layer, which, arr):
+        arr = np.ascontiguousarray(arr, np.float16)
+        rc = self.drv.homBertUpload(self.h, layer, which, arr.ctypes.data_as(ctypes.c_void_p), arr.size)
+        assert rc == 0, f"upload failed ({rc})"
+
+    def load(self, model):
+        """model: dict from synth.bert_encoder().  Weights are [K, N]; the nvte
+        path wants them as [N, K], which the compiler would transpose at compile
+        time (HOMNVGPULegalizeGemmPass)."""
+        tr = (lambda w: w.T) if self.gemm_mode == 0 else (lambda w: w)
+        for l, w in enumerate(model["weights"]):
+            for which, key in enumerate(("wqkv", "wo", "w1", "w2")):
+                self._upload(l, which, tr(w[key]))
+        self._upload(0, 4, model["word"])
+        self._upload(0, 5, model["pos_type"])
+
+    def set_inputs(self, ids=None, mask=None, hidden=None):
+        p = lambda a, dt: (np.ascontiguousarray(a, dt).ctypes.data_as(ctypes.c_void_p)
+                           if a is not None else None)
+        keep = [np.ascontiguousarray(a, dt) if a is not None else None
+                for a, dt in ((ids, np.int64), (mask, np.int64), (hidden, np.float16))]
+        ptrs = [a.ctypes.data_as(ctypes.c_void_p) if a is not None else None for a in keep]
+        assert self.drv.homBertSetInputs(self.h, *ptrs) == 0
+
+    def forward(self, from_ids=True):
+        self.drv.homBertForward(self.h, int(from_ids))
+
+    def capture(self, from_ids=True):
+        assert self.drv.homBertCapture(self.h, int(from_ids)) == 0
+
+    def replay(self):
+        assert self.drv.homBertReplay(self.h) == 0
+
+    def output(self):
+        d = self.dims
+        out = np.empty((d["bs"], d["seq"], d["hidden"]), np.float16)
+        assert self.drv.homBertGetOutput(self.h, out.ctypes.data_as(ctypes.c_void_p)) == 0
+        return out
+
+    def time(self, steps, warmup, graph=True, from_ids=True):
+        ms = self.drv.homBertTime(self.h, steps, warmup, int(graph), int(from_ids))
+        assert ms > 0, "timing failed"
+        return ms
+
+    def gemm_choices(self):
+        buf = (ctypes.c_int32 * 8)()
+        self.drv.homBertGetGemmChoices(self.h, buf)
+        names = ("qkv", "out", "ffn1", "ffn2")
+        return {n: (buf[2 * i], buf[2 * i + 1]) for i, n in enumerate(names)}

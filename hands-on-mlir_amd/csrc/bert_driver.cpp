@@ -1,0 +1,573 @@
+// Host driver for a lowered BERT encoder: the stand-in for the code that
+// hands-on-opt generates (`_hom_ciface_forward` plus its `_initFn`) and for the
+// reference's ExecutionEngine (lib/ExecutionEngine/ExecutionEngine.cpp:73-97,
+// examples/torch/bert/bert.cu:81-127).
+//
+// init:    every weight and every intermediate is allocated ONCE through the
+//          library's alloc* entry points (what ExtractInitFunc hoists,
+//          lib/Conversions/Function/ExtractInitFunc.cpp:94-188);
+// forward: a straight-line list of C-ABI calls, no host control flow and no
+//          synchronisation -- the list in HOMNVGPUToFunc.cpp for
+//            cu_seqlens; gather + add + layernorm (embeddings);
+//            per layer: QKV GEMM, attention, out-proj GEMM (+residual, in
+//            place), layernorm, FFN1 GEMM+GELU, FFN2 GEMM (+residual, in
+//            place), layernorm.
+// Because that list is static, the driver can also capture it once into a HIP
+// graph and replay it, which removes the per-call launch overhead that
+// dominates at batch 8 x seq 128.
+//
+// Everything goes through the extern "C" boundary; nothing here reaches into
+// the library's internals.
+#include "hom_amdgpu_runner_utils.h"
+
+#include <hip/hip_runtime.h>
+
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <vector>
+
+#define DRV_EXPORT extern "C" __attribute__((visibility("default")))
+
+namespace {
+
+struct Tensor {
+  C_UnrankedMemRefType m{0, nullptr};
+  void *data() const { return m.descriptor ? hom_memref_data(m.descriptor) : nullptr; }
+  void release() {
+    if (m.descriptor) {
+      deallocNVGPUF16(m.rank, m.descriptor);
+      free(m.descriptor);
+      m.descriptor = nullptr;
+    }
+  }
+};
+
+struct LayerWeights {
+  Tensor wqkv, wo, w1, w2; // [1,K,N] (manifest path) or [1,N,K] (nvte path)
+};
+
+struct GemmChoice {
+  int32_t gemmNum = 0; // 1-based manifest index, 0 = library picks
+  int32_t splitK = 1;
+};
+
+} // namespace
+
+struct HomBertEncoder {
+  int layers, hidden, heads, ffn, batch, seq, vocab;
+  int gemmMode; // 0 = nvteGemmF16 (B pre-transposed), 1 = cutlassGemmF16 +
+                // tuned table / heuristic, 2 = cutlassGemmF16 + live autotune
+  int geluForm; // 0 erf, 1 tanh (manifest path only; nvte path is tanh)
+  float eps;
+  std::vector<LayerWeights> w;
+  Tensor wordEmb;   // [1, vocab, H]
+  Tensor posType;   // [1, seq, H]  (position + token-type rows, constant folded)
+  Tensor ids;       // int64 [b, s]   (descriptor built by hand, see create)
+  Tensor mask;      // int64 [b, s]
+  Tensor cu;        // int32 [b+1]
+  Tensor h, emb, qkv, attn, f;
+  GemmChoice cQkv, cOut, cFfn1, cFfn2;
+  hipStream_t stream = nullptr;
+  hipGraph_t graph = nullptr;
+  hipGraphExec_t graphExec = nullptr;
+  hipEvent_t evStart = nullptr, evStop = nullptr;
+};
+
+namespace {
+
+bool hipOk(hipError_t e, const char *what) {
+  if (e != hipSuccess) {
+    fprintf(stderr, "hom_bert_driver: %s failed: %s\n", what,
+            hipGetErrorString(e));
+    return false;
+  }
+  return true;
+}
+
+// int64 [b, s] tensor: there is no alloc entry point for it in the boundary
+// (the reference's driver builds these with allocHelper itself, bert.cu:27-78).
+Tensor allocI64_2D(int64_t a, int64_t b) {
+  Tensor t;
+  auto *d = static_cast<HomStridedMemRef2 *>(malloc(sizeof(HomStridedMemRef2)));
+  void *dev = nullptr;
+  if (!hipOk(hipMalloc(&dev, size_t(a) * b * sizeof(int64_t)), "hipMalloc")) {
+    free(d);
+    return t;
+  }
+  d->basePtr = d->data = dev;
+  d->offset = 0;
+  d->sizes[0] = a;
+  d->sizes[1] = b;
+  d->strides[0] = b;
+  d->strides[1] = 1;
+  t.m.rank = 2;
+  t.m.descriptor = d;
+  return t;
+}
+
+void gemm(HomBertEncoder *e, const Tensor &a, const Tensor &w, const Tensor &c,
+          const Tensor &d, int64_t act, float beta, const GemmChoice &ch) {
+  if (e->gemmMode == 0) {
+    nvteGemmF16(a.m.rank, a.m.descriptor, false, w.m.rank, w.m.descriptor, true,
+                c.m.rank, c.m.descriptor, d.m.rank, d.m.descriptor, act, 1.0f,
+                beta, 0, 1);
+  } else {
+    cutlassGemmF16(a.m.rank, a.m.descriptor, false, w.m.rank, w.m.descriptor,
+                   false, c.m.rank, c.m.descriptor, d.m.rank, d.m.descriptor,
+                   act, 1.0f, beta, ch.gemmNum, ch.splitK);
+  }
+}
+
+void chooseGemm(HomBertEncoder *e, int64_t M, int64_t N, int64_t K, int64_t act,
+                float beta, GemmChoice *out) {
+  int64_t idx = -1;
+  int32_t sk = 1;
+  if (e->gemmMode == 2)
+    homGemmProfile(M, N, K, act, 1.0f, beta, &idx, &sk, nullptr);
+  else
+    homGemmSelect(M, N, K, act, &idx, &sk);
+  out->gemmNum = int32_t(idx + 1);
+  out->splitK = sk;
+}
+
+void callList(HomBertEncoder *e, int fromIds) {
+  thrustCuSeqLenI64(e->mask.m.rank, e->mask.m.descriptor, e->cu.m.rank,
+                    e->cu.m.descriptor);
+  if (fromIds) {
+    thrustGatherF16(e->ids.m.rank, e->ids.m.descriptor, e->wordEmb.m.rank,
+                    e->wordEmb.m.descriptor, e->emb.m.rank,
+                    e->emb.m.descriptor);
+    thrustElementwiseAddF16(e->emb.m.rank, e->emb.m.descriptor,
+                            e->posType.m.rank, e->posType.m.descriptor,
+                            e->h.m.rank, e->h.m.descriptor);
+    nvteLayernormF16(e->h.m.rank, e->h.m.descriptor, e->eps);
+  }
+  const float scale = 1.0f / sqrtf(float(e->hidden / e->heads));
+  const int64_t geluAct = e->gemmMode == 0 ? 1 : (e->geluForm == 1 ? 2 : 1);
+  for (int l = 0; l < e->layers; l++) {
+    const LayerWeights &w = e->w[l];
+    gemm(e, e->h, w.wqkv, e->qkv, e->qkv, 0, 0.0f, e->cQkv);
+    nvteBertAttentionF16(e->qkv.m.rank, e->qkv.m.descriptor, e->cu.m.rank,
+                         e->cu.m.descriptor, e->attn.m.rank,
+                         e->attn.m.descriptor, scale, e->heads);
+    gemm(e, e->attn, w.wo, e->h, e->h, 0, 1.0f, e->cOut);
+    nvteLayernormF16(e->h.m.rank, e->h.m.descriptor, e->eps);
+    gemm(e, e->h, w.w1, e->f, e->f, geluAct, 0.0f, e->cFfn1);
+    gemm(e, e->f, w.w2, e->h, e->h, 0, 1.0f, e->cFfn2);
+    nvteLayernormF16(e->h.m.rank, e->h.m.descriptor, e->eps);
+  }
+}
+
+} // namespace
+
+// gemmMode / geluForm as documented on HomBertEncoder.
+DRV_EXPORT HomBertEncoder *homBertCreate(int layers, int hidden, int heads,
+                                         int ffn, int batch, int seq, int vocab,
+                                         int gemmMode, int geluForm) {
+  auto *e = new HomBertEncoder();
+  e->layers = layers;
+  e->hidden = hidden;
+  e->heads = heads;
+  e->ffn = ffn;
+  e->batch = batch;
+  e->seq = seq;
+  e->vocab = vocab;
+  e->gemmMode = gemmMode;
+  e->geluForm = geluForm;
+  e->eps = 1e-12f;
+  e->w.resize(size_t(layers));
+  const bool nk = gemmMode == 0;
+  for (auto &w : e->w) {
+    w.wqkv.m = nk ? alloc3DMemRefNVGPUF16(1, 3 * hidden, hidden)
+                  : alloc3DMemRefNVGPUF16(1, hidden, 3 * hidden);
+    w.wo.m = alloc3DMemRefNVGPUF16(1, hidden, hidden);
+    w.w1.m = nk ? alloc3DMemRefNVGPUF16(1, ffn, hidden)
+                : alloc3DMemRefNVGPUF16(1, hidden, ffn);
+    w.w2.m = nk ? alloc3DMemRefNVGPUF16(1, hidden, ffn)
+                : alloc3DMemRefNVGPUF16(1, ffn, hidden);
+  }
+  e->wordEmb.m = alloc3DMemRefNVGPUF16(1, vocab, hidden);
+  e->posType.m = alloc3DMemRefNVGPUF16(1, seq, hidden);
+  e->ids = allocI64_2D(batch, seq);
+  e->mask = allocI64_2D(batch, seq);
+  e->cu.m = alloc1DMemRefNVGPUI32(batch + 1);
+  e->h.m = alloc3DMemRefNVGPUF16(batch, seq, hidden);
+  e->emb.m = alloc3DMemRefNVGPUF16(batch, seq, hidden);
+  e->qkv.m = alloc3DMemRefNVGPUF16(batch, seq, 3 * hidden);
+  e->attn.m = alloc3DMemRefNVGPUF16(batch, seq, hidden);
+  e->f.m = alloc3DMemRefNVGPUF16(batch, seq, ffn);
+  if (!hipOk(hipStreamCreateWithFlags(&e->stream, hipStreamNonBlocking),
+             "hipStreamCreate") ||
+      !hipOk(hipEventCreate(&e->evStart), "hipEventCreate") ||
+      !hipOk(hipEventCreate(&e->evStop), "hipEventCreate"))
+    return e;
+  if (gemmMode != 0) {
+    const int64_t M = int64_t(batch) * seq;
+    const int64_t gelu = geluForm == 1 ? 2 : 1;
+    chooseGemm(e, M, 3 * hidden, hidden, 0, 0.0f, &e->cQkv);
+    chooseGemm(e, M, hidden, hidden, 0, 1.0f, &e->cOut);
+    chooseGemm(e, M, ffn, hidden, gelu, 0.0f, &e->cFfn1);
+    chooseGemm(e, M, hidden, ffn, 0, 1.0f, &e->cFfn2);
+  }
+  return e;
+}
+
+DRV_EXPORT void homBertDestroy(HomBertEncoder *e) {
+  if (!e)
+    return;
+  if (e->graphExec)
+    (void)hipGraphExecDestroy(e->graphExec);
+  if (e->graph)
+    (void)hipGraphDestroy(e->graph);
+  if (e->stream) {
+    (void)hipStreamSynchronize(e->stream);
+    (void)hipStreamDestroy(e->stream);
+  }
+  if (e->evStart)
+    (void)hipEventDestroy(e->evStart);
+  if (e->evStop)
+    (void)hipEventDestroy(e->evStop);
+  for (auto &w : e->w) {
+    w.wqkv.release();
+    w.wo.release();
+    w.w1.release();
+    w.w2.release();
+  }
+  for (Tensor *t : {&e->wordEmb, &e->posType, &e->ids, &e->mask, &e->cu, &e->h,
+                    &e->emb, &e->qkv, &e->attn, &e->f})
+    t->release();
+  delete e;
+}
+
+// which: 0 Wqkv, 1 Wo, 2 W1, 3 W2 (layer >= 0); 4 word embeddings, 5 position +
+// token-type rows (layer ignored).  `host` holds fp16 values in the layout the
+// tensor was allocated with ([K, N] row-major, or [N, K] when gemmMode == 0).
+DRV_EXPORT int homBertUpload(HomBertEncoder *e, int layer, int which,
+                             const void *host, int64_t numel) {
+  Tensor *t = nullptr;
+  if (which <= 3) {
+    if (layer < 0 || layer >= e->layers)
+      return -1;
+    LayerWeights &w = e->w[size_t(layer)];
+    t = which == 0 ? &w.wqkv : which == 1 ? &w.wo : which == 2 ? &w.w1 : &w.w2;
+  } else {
+    t = which == 4 ? &e->wordEmb : &e->posType;
+  }
+  int64_t expect = 1;
+  for (int64_t i = 0; i < t->m.rank; i++)
+    expect *= hom_memref_sizes(t->m.descriptor)[i];
+  if (expect != numel) {
+    fprintf(stderr, "hom_bert_driver: upload of %lld values into a tensor of "
+                    "%lld\n", (long long)numel, (long long)expect);
+    return -2;
+  }
+  return hipOk(hipMemcpy(t->data(), host, size_t(numel) * 2,
+                         hipMemcpyHostToDevice),
+               "hipMemcpy")
+             ? 0
+             : -3;
+}
+
+// Inputs: token ids and 0/1 mask (int64 [b, s]); `hidden` (fp16 [b, s, H]) may
+// be given instead of ids to start from precomputed embeddings.
+DRV_EXPORT int homBertSetInputs(HomBertEncoder *e, const int64_t *ids,
+                                const int64_t *mask, const void *hidden) {
+  const size_t n = size_t(e->batch) * e->seq;
+  if (ids && !hipOk(hipMemcpy(e->ids.data(), ids, n * 8, hipMemcpyHostToDevice),
+                    "hipMemcpy ids"))
+    return -1;
+  if (mask &&
+      !hipOk(hipMemcpy(e->mask.data(), mask, n * 8, hipMemcpyHostToDevice),
+             "hipMemcpy mask"))
+    return -1;
+  if (hidden && !hipOk(hipMemcpy(e->h.data(), hidden, n * e->hidden * 2,
+                                 hipMemcpyHostToDevice),
+                       "hipMemcpy hidden"))
+    return -1;
+  return 0;
+}
+
+// One eager forward on the driver's stream; returns after enqueueing.
+DRV_EXPORT void homBertForward(HomBertEncoder *e, int fromIds) {
+  void *prev = homGetStream();
+  homSetStream(e->stream);
+  callList(e, fromIds);
+  homSetStream(prev);
+}
+
+// Capture the call list once (after one eager run has sized the library's
+// scratch buffers) and keep the instantiated graph.
+DRV_EXPORT int homBertCapture(HomBertEncoder *e, int fromIds) {
+  homBertForward(e, fromIds);
+  if (!hipOk(hipStreamSynchronize(e->stream), "hipStreamSynchronize"))
+    return -1;
+  if (e->graphExec) {
+    (void)hipGraphExecDestroy(e->graphExec);
+    e->graphExec = nullptr;
+  }
+  if (e->graph) {
+    (void)hipGraphDestroy(e->graph);
+    e->graph = nullptr;
+  }
+  void *prev = homGetStream();
+  homSetStream(e->stream);
+  bool ok = hipOk(hipStreamBeginCapture(e->stream, hipStreamCaptureModeRelaxed),
+                  "hipStreamBeginCapture");
+  if (ok) {
+    callList(e, fromIds);
+    ok = hipOk(hipStreamEndCapture(e->stream, &e->graph), "hipStreamEndCapture");
+  }
+  homSetStream(prev);
+  if (!ok)
+    return -1;
+  if (!hipOk(hipGraphInstantiate(&e->graphExec, e->graph, nullptr, nullptr, 0),
+             "hipGraphInstantiate"))
+    return -1;
+  return 0;
+}
+
+DRV_EXPORT int homBertReplay(HomBertEncoder *e) {
+  if (!e->graphExec)
+    return -1;
+  return hipOk(hipGraphLaunch(e->graphExec, e->stream), "hipGraphLaunch") ? 0
+                                                                          : -1;
+}
+
+DRV_EXPORT int homBertSync(HomBertEncoder *e) {
+  return hipOk(hipStreamSynchronize(e->stream), "hipStreamSynchronize") ? 0 : -1;
+}
+
+// Copy the encoder output (the hidden-state buffer, updated in place) to host.
+DRV_EXPORT int homBertGetOutput(HomBertEncoder *e, void *host) {
+  if (homBertSync(e) != 0)
+    return -1;
+  const size_t n = size_t(e->batch) * e->seq * e->hidden;
+  return hipOk(hipMemcpy(host, e->h.data(), n * 2, hipMemcpyDeviceToHost),
+               "hipMemcpy out")
+             ? 0
+             : -1;
+}
+
+// Time `steps` forwards after `warmup` untimed ones, bracketed by events on the
+// driver's stream (the reference's protocol: bert.cu:95-127).  useGraph != 0
+// replays the captured graph.  Returns mean milliseconds per forward, < 0 on
+// error.  Inputs stay resident; every forward recomputes from the token ids.
+DRV_EXPORT double homBertTime(HomBertEncoder *e, int steps, int warmup,
+                              int useGraph, int fromIds) {
+  if (useGraph && !e->graphExec && homBertCapture(e, fromIds) != 0)
+    return -1.0;
+  for (int i = 0; i < warmup; i++) {
+    if (useGraph)
+      homBertReplay(e);
+    else
+      homBertForward(e, fromIds);
+  }
+  if (homBertSync(e) != 0)
+    return -1.0;
+  (void)hipEventRecord(e->evStart, e->stream);
+  for (int i = 0; i < steps; i++) {
+    if (useGraph)
+      homBertReplay(e);
+    else
+      homBertForward(e, fromIds);
+  }
+  (void)hipEventRecord(e->evStop, e->stream);
+  if (!hipOk(hipEventSynchronize(e->evStop), "hipEventSynchronize"))
+    return -1.0;
+  float ms = 0.f;
+  (void)hipEventElapsedTime(&ms, e->evStart, e->evStop);
+  return double(ms) / double(steps > 0 ? steps : 1);
+}
+
+DRV_EXPORT void homBertGetGemmChoices(HomBertEncoder *e, int32_t *out8) {
+  const GemmChoice *c[4] = {&e->cQkv, &e->cOut, &e->cFfn1, &e->cFfn2};
+  for (int i = 0; i < 4; i++) {
+    out8[2 * i] = c[i]->gemmNum;
+    out8[2 * i + 1] = c[i]->splitK;
+  }
+}
+
+// ---- single-operator timing through the boundary -------------------------
+// Each helper enqueues `iters` back-to-back calls of one entry point between
+// two events on a private stream and returns mean milliseconds per call.
+
+namespace {
+struct Timer {
+  hipStream_t s = nullptr;
+  hipEvent_t a = nullptr, b = nullptr;
+  void *prev = nullptr;
+  bool ok = false;
+  Timer() {
+    ok = hipOk(hipStreamCreateWithFlags(&s, hipStreamNonBlocking), "stream") &&
+         hipOk(hipEventCreate(&a), "event") && hipOk(hipEventCreate(&b), "event");
+    prev = homGetStream();
+    homSetStream(s);
+  }
+  ~Timer() {
+    homSetStream(prev);
+    if (a)
+      (void)hipEventDestroy(a);
+    if (b)
+      (void)hipEventDestroy(b);
+    if (s) {
+      (void)hipStreamSynchronize(s);
+      (void)hipStreamDestroy(s);
+    }
+  }
+  template <typename F> double run(F &&fn, int iters, int warmup) {
+    if (!ok)
+      return -1.0;
+    for (int i = 0; i < warmup; i++)
+      fn();
+    if (!hipOk(hipStreamSynchronize(s), "sync"))
+      return -1.0;
+    (void)hipEventRecord(a, s);
+    for (int i = 0; i < iters; i++)
+      fn();
+    (void)hipEventRecord(b, s);
+    if (!hipOk(hipEventSynchronize(b), "event sync"))
+      return -1.0;
+    float ms = 0.f;
+    (void)hipEventElapsedTime(&ms, a, b);
+    return double(ms) / double(iters > 0 ? iters : 1);
+  }
+};
+
+void fillRandomF16(void *dev, int64_t numel, float scale, uint32_t seed) {
+  std::vector<uint16_t> host(static_cast<size_t>(numel));
+  uint32_t x = seed * 2654435761u + 12345u;
+  for (auto &v : host) {
+    // xorshift; sum of 4 uniforms, roughly normal, scaled
+    float acc = 0.f;
+    for (int i = 0; i < 4; i++) {
+      x ^= x << 13;
+      x ^= x >> 17;
+      x ^= x << 5;
+      acc += float(x & 0xffff) / 65536.0f - 0.5f;
+    }
+    _Float16 h = _Float16(acc * 1.7320508f * scale);
+    memcpy(&v, &h, 2);
+  }
+  (void)hipMemcpy(dev, host.data(), size_t(numel) * 2, hipMemcpyHostToDevice);
+}
+} // namespace
+
+// D = act(A.B + bias) with bias broadcast as a [1,1,N] C (useBias) or beta = 0.
+// gemmNum is 1-based (0 = library picks); returns ms per call.
+DRV_EXPORT double homTimeGemm(int64_t M, int64_t N, int64_t K, int64_t act,
+                              int useBias, int32_t gemmNum, int32_t splitK,
+                              int iters, int warmup) {
+  Tensor a, b, c, d;
+  a.m = alloc3DMemRefNVGPUF16(1, int32_t(M), int32_t(K));
+  b.m = alloc3DMemRefNVGPUF16(1, int32_t(K), int32_t(N));
+  c.m = alloc3DMemRefNVGPUF16(1, 1, int32_t(N));
+  d.m = alloc3DMemRefNVGPUF16(1, int32_t(M), int32_t(N));
+  fillRandomF16(a.data(), M * K, 1.0f, 1);
+  fillRandomF16(b.data(), K * N, 0.02f, 2);
+  fillRandomF16(c.data(), N, 0.02f, 3);
+  double ms;
+  {
+    Timer t;
+    ms = t.run(
+        [&] {
+          cutlassGemmF16(3, a.m.descriptor, false, 3, b.m.descriptor, false, 3,
+                         useBias ? c.m.descriptor : d.m.descriptor, 3,
+                         d.m.descriptor, act, 1.0f, useBias ? 1.0f : 0.0f,
+                         gemmNum, splitK);
+        },
+        iters, warmup);
+  }
+  a.release();
+  b.release();
+  c.release();
+  d.release();
+  return ms;
+}
+
+// In-place layer norm (reference form) when fused == 0; residual add + affine
+// layer norm (homAddLayernormF16) when fused != 0.
+DRV_EXPORT double homTimeLayernorm(int64_t rows, int64_t hidden, int fused,
+                                   int iters, int warmup) {
+  Tensor x, r, g, bt, o;
+  x.m = alloc3DMemRefNVGPUF16(1, int32_t(rows), int32_t(hidden));
+  r.m = alloc3DMemRefNVGPUF16(1, int32_t(rows), int32_t(hidden));
+  o.m = alloc3DMemRefNVGPUF16(1, int32_t(rows), int32_t(hidden));
+  g.m = alloc3DMemRefNVGPUF16(1, 1, int32_t(hidden));
+  bt.m = alloc3DMemRefNVGPUF16(1, 1, int32_t(hidden));
+  fillRandomF16(x.data(), rows * hidden, 1.0f, 4);
+  fillRandomF16(r.data(), rows * hidden, 1.0f, 5);
+  fillRandomF16(g.data(), hidden, 0.02f, 6);
+  fillRandomF16(bt.data(), hidden, 0.02f, 7);
+  double ms;
+  {
+    Timer t;
+    ms = t.run(
+        [&] {
+          if (fused)
+            homAddLayernormF16(3, x.m.descriptor, 3, r.m.descriptor, 3,
+                               g.m.descriptor, 3, bt.m.descriptor, 3,
+                               o.m.descriptor, 1e-12f);
+          else
+            nvteLayernormF16(3, x.m.descriptor, 1e-12f);
+        },
+        iters, warmup);
+  }
+  for (Tensor *t : {&x, &r, &g, &bt, &o})
+    t->release();
+  return ms;
+}
+
+// Packed-QKV attention with per-sequence valid lengths `lens` (host, int32[bs]).
+DRV_EXPORT double homTimeAttention(int64_t bs, int64_t seq, int64_t heads,
+                                   const int32_t *lens, int iters, int warmup) {
+  const int64_t hd = heads * 64;
+  Tensor qkv, out, cu;
+  qkv.m = alloc3DMemRefNVGPUF16(int32_t(bs), int32_t(seq), int32_t(3 * hd));
+  out.m = alloc3DMemRefNVGPUF16(int32_t(bs), int32_t(seq), int32_t(hd));
+  cu.m = alloc1DMemRefNVGPUI32(int32_t(bs + 1));
+  fillRandomF16(qkv.data(), bs * seq * 3 * hd, 1.0f, 8);
+  std::vector<int32_t> cuHost(size_t(bs + 1), 0);
+  for (int64_t i = 0; i < bs; i++)
+    cuHost[size_t(i + 1)] = cuHost[size_t(i)] + lens[i];
+  (void)hipMemcpy(cu.data(), cuHost.data(), size_t(bs + 1) * 4,
+                  hipMemcpyHostToDevice);
+  double ms;
+  {
+    Timer t;
+    ms = t.run(
+        [&] {
+          nvteBertAttentionF16(3, qkv.m.descriptor, 1, cu.m.descriptor, 3,
+                               out.m.descriptor, 0.125f, heads);
+        },
+        iters, warmup);
+  }
+  qkv.release();
+  out.release();
+  cu.release();
+  return ms;
+}
+
+DRV_EXPORT double homTimeElementwiseAdd(int64_t rows, int64_t hidden, int iters,
+                                        int warmup) {
+  Tensor a, b, o;
+  a.m = alloc3DMemRefNVGPUF16(1, int32_t(rows), int32_t(hidden));
+  b.m = alloc3DMemRefNVGPUF16(1, int32_t(rows), int32_t(hidden));
+  o.m = alloc3DMemRefNVGPUF16(1, int32_t(rows), int32_t(hidden));
+  fillRandomF16(a.data(), rows * hidden, 1.0f, 9);
+  fillRandomF16(b.data(), rows * hidden, 1.0f, 10);
+  double ms;
+  {
+    Timer t;
+    ms = t.run(
+        [&] {
+          thrustElementwiseAddF16(3, a.m.descriptor, 3, b.m.descriptor, 3,
+                                  o.m.descriptor);
+        },
+        iters, warmup);
+  }
+  a.release();
+  b.release();
+  o.release();
+  return ms;
+}

@@ -1,0 +1,104 @@
+// Shared host-side plumbing for the runtime kernel library: argument checks,
+// HIP error handling, the library stream, memref views and grow-only device
+// scratch.  Plays the role of include/NVGPUKernels/Utils.h:45-52,179-238 in
+// the reference (checkCudaErrors, getDummyPointer, getMulitProcessorCount).
+#pragma once
+
+#include "hom_memref.h"
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <string>
+
+namespace hom {
+
+// ---------------------------------------------------------------- errors --
+// mode 0: print + abort (reference behaviour); mode 1: print, remember, and
+// let the entry point return early.
+int errorMode();
+void setErrorMode(int mode);
+void recordError(const char *file, int line, const char *fmt, ...)
+    __attribute__((format(printf, 3, 4)));
+const char *takeLastError();
+
+// Check an argument condition inside a void entry point / runner.  On failure
+// either aborts or returns `ret` from the enclosing function.
+#define HOM_CHECK_RET(cond, ret, ...)                                          \
+  do {                                                                         \
+    if (!(cond)) {                                                             \
+      ::hom::recordError(__FILE__, __LINE__, __VA_ARGS__);                     \
+      return ret;                                                              \
+    }                                                                          \
+  } while (0)
+
+#define HOM_HIP_RET(expr, ret)                                                 \
+  do {                                                                         \
+    hipError_t _e = (expr);                                                    \
+    if (_e != hipSuccess) {                                                    \
+      ::hom::recordError(__FILE__, __LINE__, "HIP error %d (%s) from %s",      \
+                         int(_e), hipGetErrorString(_e), #expr);               \
+      return ret;                                                              \
+    }                                                                          \
+  } while (0)
+
+enum class Status : int { kSuccess = 0, kInvalidArgument = 1, kInternal = 2 };
+
+// ---------------------------------------------------------------- stream --
+hipStream_t stream();
+void setStream(hipStream_t s);
+
+// ------------------------------------------------------------ memref view --
+// Equivalent of convertToDynamicMemRefType (HandsOnRunnerUtils.h:37-42): reads
+// `data`, `sizes`, `strides`; `offset` is ignored exactly as the reference's
+// runners ignore it (e.g. GemmRunner.h:279-284 passes A.data directly).
+template <typename T> struct View {
+  int64_t rank = 0;
+  T *data = nullptr;
+  const int64_t *sizes = nullptr;
+  const int64_t *strides = nullptr;
+
+  View() = default;
+  View(int64_t rank_, void *descriptor) : rank(rank_) {
+    if (descriptor) {
+      data = static_cast<T *>(static_cast<HomMemRefHeader *>(descriptor)->data);
+      sizes = hom_memref_sizes(descriptor);
+      strides = hom_memref_strides(descriptor, rank_);
+    }
+  }
+  int64_t numel() const {
+    int64_t n = 1;
+    for (int64_t i = 0; i < rank; i++)
+      n *= sizes[i];
+    return n;
+  }
+  bool contiguous() const {
+    int64_t expect = 1;
+    for (int64_t i = rank - 1; i >= 0; i--) {
+      if (sizes[i] != 1 && strides[i] != expect)
+        return false;
+      expect *= sizes[i];
+    }
+    return true;
+  }
+};
+
+// ---------------------------------------------------------------- device --
+struct DeviceInfo {
+  int computeUnits = 0;
+  int clockKHz = 0;
+  size_t l2Bytes = 0;
+};
+const DeviceInfo &deviceInfo();
+
+// Grow-only device scratch, one buffer per slot.  Slot kWorkspace holds
+// split-K partial tiles, kCounters the per-tile arrival counters (kept zero
+// between launches by the kernels themselves), kTemp short-lived temporaries.
+enum ScratchSlot { kWorkspace = 0, kCounters = 1, kTemp = 2, kNumSlots = 3 };
+// Returns nullptr (after recording an error) on allocation failure.  `zero`
+// clears newly allocated memory once, at allocation time.
+void *scratch(ScratchSlot slot, size_t bytes, bool zero);
+
+} // namespace hom

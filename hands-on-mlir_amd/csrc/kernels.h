@@ -1,0 +1,95 @@
+// Launch interfaces of the HIP kernels (device pointers + plain sizes).  The
+// runners in runners.cpp validate memref arguments and call these.
+#pragma once
+
+#include "common.h"
+
+namespace hom {
+
+// ------------------------------------------------------------- layernorm --
+// out[r, :] = ((x[r,:] (+ res[r,:])) - mean) * rstd (* gamma + beta).
+// T is _Float16 or float.  res/gamma/beta may be null.  out may alias x.
+template <typename T>
+Status launchLayernorm(const T *x, const T *res, const T *gamma, const T *beta,
+                       T *out, int64_t rows, int64_t hidden, float eps,
+                       hipStream_t s);
+
+// ----------------------------------------------------------- elementwise --
+enum class BinOp : int { kAdd = 0, kSub = 1, kMul = 2, kDiv = 3 };
+constexpr int kMaxRank = 8;
+struct BroadcastDesc {
+  int rank;
+  int64_t outSize[kMaxRank];
+  int64_t outStride[kMaxRank]; // contiguous strides of A/Out
+  int64_t bSize[kMaxRank];
+  int64_t bStride[kMaxRank];
+};
+template <typename T>
+Status launchElementwise(BinOp op, const T *a, const T *b, T *out,
+                         int64_t total, const BroadcastDesc &desc,
+                         hipStream_t s);
+
+template <typename T>
+Status launchGather(const int64_t *indices, const T *value, T *out,
+                    int64_t numIndices, int64_t vocab, int64_t rowLength,
+                    hipStream_t s);
+
+template <typename InT>
+Status launchCuSeqLen(const InT *mask, int32_t *out, int64_t bs, int64_t seq,
+                      hipStream_t s);
+
+Status launchGeluF16(const _Float16 *in, _Float16 *out, int64_t total, int form,
+                     hipStream_t s);
+
+// Per-row statistics of a [rows, n] fp16 matrix in the form the LN-GEMM pair
+// exchanges: var[r] = 1/sqrt(E[x^2]-E[x]^2+eps), mean[r] = -E[x]*var[r].
+Status launchRowStatsF16(const _Float16 *d, _Float16 *var, _Float16 *mean,
+                         int64_t rows, int64_t n, float eps, hipStream_t s);
+// out[r, k] = a[r, k] * var[r] + mean[r]  (fp32 math, fp16 store).
+Status launchApplyRowStatsF16(const _Float16 *a, const _Float16 *var,
+                              const _Float16 *mean, _Float16 *out, int64_t rows,
+                              int64_t k, hipStream_t s);
+
+// ------------------------------------------------------------- attention --
+// qkv [bs, seq, 3*heads*headDim] fp16, cu int32[bs+1], out [bs, seq,
+// heads*headDim].  headDim must be 64.
+Status launchBertAttentionF16(const _Float16 *qkv, const int32_t *cuSeqlens,
+                              _Float16 *out, int64_t bs, int64_t seq,
+                              int64_t heads, int64_t headDim, float scale,
+                              hipStream_t s);
+
+// ------------------------------------------------------------------ gemm --
+enum class Epilogue : int { kLinear = 0, kGeluErf = 1, kGeluTanh = 2 };
+
+struct GemmProblem {
+  const _Float16 *A; // [M, K], row stride lda
+  const _Float16 *B; // [K, N] row-major (bIsNK false) or [N, K] (bIsNK true)
+  const _Float16 *C; // may be null when beta == 0
+  _Float16 *D;
+  int64_t M, N, K;
+  int64_t lda, ldb, ldd;
+  // Source addressing: C[(row % cRowPeriod) * ldc + col]; cRowPeriod == M for a
+  // full matrix, 1 for a bias row, M' for a per-batch broadcast.  ldc == 0 for
+  // a bias row.
+  int64_t ldc;
+  int64_t cRowPeriod;
+  float alpha, beta;
+  bool bIsNK;
+  int splitK;
+};
+
+struct GemmKernelInfo {
+  const char *name;
+  int tileM, tileN, tileK;
+  int wavesM, wavesN;
+  int alignment; // required divisor of N and K (8 or 1)
+  int activation; // 0 linear, 1 gelu (what the profiler filters on)
+  Epilogue epilogue;
+};
+
+int gemmKernelCount();
+const GemmKernelInfo &gemmKernelInfo(int idx);
+// Validates alignment/split-K against the kernel and launches it.
+Status launchGemm(int idx, const GemmProblem &p, hipStream_t s);
+
+} // namespace hom

@@ -1,0 +1,254 @@
+// Layer norm over the last dimension for gfx950.
+//
+// Semantics follow the reference's LayernormRunner (include/NVGPUKernels/
+// Layernorm.h:584-694): statistics in fp32, biased variance, y = (x - mean) *
+// rsqrt(var + eps); the reference form has no affine parameters and runs in
+// place.  The optional residual / gamma / beta operands are a superset.
+//
+// The kernel is bandwidth bound: each row is read once with 128-bit loads and
+// stays in registers for the two statistic passes; one 64-lane wavefront owns
+// a row and reduces with cross-lane shuffles (no LDS).  Rows that do not fit
+// that scheme (odd lengths, very long rows) take a workgroup-per-row kernel
+// that reduces through LDS.
+#include "kernels.h"
+
+namespace hom {
+namespace {
+
+constexpr int kWave = 64;
+
+template <typename T> struct Vec16;
+template <> struct Vec16<_Float16> {
+  static constexpr int kN = 8;
+  typedef _Float16 type __attribute__((ext_vector_type(8)));
+};
+template <> struct Vec16<float> {
+  static constexpr int kN = 4;
+  typedef float type __attribute__((ext_vector_type(4)));
+};
+
+__device__ __forceinline__ float waveSum(float v) {
+#pragma unroll
+  for (int off = kWave / 2; off > 0; off >>= 1)
+    v += __shfl_xor(v, off, kWave);
+  return v;
+}
+
+// One wavefront per row; VPL 16-byte vectors per lane.
+template <typename T, int VPL, bool HAS_RES, bool HAS_AFFINE>
+__global__ __launch_bounds__(256) void layernormWaveKernel(
+    const T *x, const T *res,
+    const T *__restrict__ gamma, const T *__restrict__ beta, T *out,
+    int64_t rows, int hidden, float eps) {
+  using V = typename Vec16<T>::type;
+  constexpr int N = Vec16<T>::kN;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t row = int64_t(blockIdx.x) * (blockDim.x / kWave) +
+                      (threadIdx.x / kWave);
+  if (row >= rows)
+    return;
+  const int nvec = hidden / N;
+  const V *xr = reinterpret_cast<const V *>(x + row * hidden);
+  const V *rr = HAS_RES ? reinterpret_cast<const V *>(res + row * hidden)
+                        : nullptr;
+
+  float v[VPL][N];
+  V raw[VPL];
+  V rawRes[VPL];
+#pragma unroll
+  for (int i = 0; i < VPL; i++) {
+    const int idx = lane + i * kWave;
+    if (idx < nvec) {
+      raw[i] = xr[idx];
+      if (HAS_RES)
+        rawRes[i] = rr[idx];
+    }
+  }
+  float sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < VPL; i++) {
+    const int idx = lane + i * kWave;
+#pragma unroll
+    for (int j = 0; j < N; j++) {
+      float f = 0.f;
+      if (idx < nvec) {
+        f = float(raw[i][j]);
+        if (HAS_RES)
+          f += float(rawRes[i][j]); // the sum stays in fp32
+      }
+      v[i][j] = f;
+      sum += f;
+    }
+  }
+  const float invH = 1.0f / float(hidden);
+  const float mean = waveSum(sum) * invH;
+  float sq = 0.f;
+#pragma unroll
+  for (int i = 0; i < VPL; i++) {
+    const int idx = lane + i * kWave;
+    if (idx < nvec) {
+#pragma unroll
+      for (int j = 0; j < N; j++) {
+        const float d = v[i][j] - mean;
+        sq += d * d;
+      }
+    }
+  }
+  const float var = waveSum(sq) * invH;
+  const float rstd = 1.0f / sqrtf(var + eps);
+
+  V *orow = reinterpret_cast<V *>(out + row * hidden);
+#pragma unroll
+  for (int i = 0; i < VPL; i++) {
+    const int idx = lane + i * kWave;
+    if (idx < nvec) {
+      V o;
+      if (HAS_AFFINE) {
+        V g, b;
+        bool hasG = gamma != nullptr, hasB = beta != nullptr;
+        if (hasG)
+          g = reinterpret_cast<const V *>(gamma)[idx];
+        if (hasB)
+          b = reinterpret_cast<const V *>(beta)[idx];
+#pragma unroll
+        for (int j = 0; j < N; j++) {
+          float y = (v[i][j] - mean) * rstd;
+          if (hasG)
+            y *= float(g[j]);
+          if (hasB)
+            y += float(b[j]);
+          o[j] = T(y);
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < N; j++)
+          o[j] = T((v[i][j] - mean) * rstd);
+      }
+      orow[idx] = o;
+    }
+  }
+}
+
+__device__ __forceinline__ float blockSum(float v, float *lds) {
+  v = waveSum(v);
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const int nwaves = blockDim.x / kWave;
+  __syncthreads(); // lds may still be read from a previous reduction
+  if (lane == 0)
+    lds[wave] = v;
+  __syncthreads();
+  float total = 0.f;
+  for (int i = 0; i < nwaves; i++)
+    total += lds[i];
+  return total;
+}
+
+// One workgroup per row, any row length, scalar accesses.
+template <typename T>
+__global__ __launch_bounds__(256) void layernormBlockKernel(
+    const T *x, const T *res,
+    const T *__restrict__ gamma, const T *__restrict__ beta, T *out,
+    int64_t rows, int64_t hidden, float eps) {
+  __shared__ float lds[8];
+  const int64_t row = blockIdx.x;
+  const T *xr = x + row * hidden;
+  const T *rr = res ? res + row * hidden : nullptr;
+  T *orow = out + row * hidden;
+  auto load = [&](int64_t i) -> float {
+    float f = float(xr[i]);
+    if (rr)
+      f += float(rr[i]);
+    return f;
+  };
+  float sum = 0.f;
+  for (int64_t i = threadIdx.x; i < hidden; i += blockDim.x)
+    sum += load(i);
+  const float mean = blockSum(sum, lds) / float(hidden);
+  float sq = 0.f;
+  for (int64_t i = threadIdx.x; i < hidden; i += blockDim.x) {
+    const float d = load(i) - mean;
+    sq += d * d;
+  }
+  const float var = blockSum(sq, lds) / float(hidden);
+  const float rstd = 1.0f / sqrtf(var + eps);
+  // All reads of this row are done (blockSum synchronised) before any write,
+  // so out may alias x.
+  for (int64_t i = threadIdx.x; i < hidden; i += blockDim.x) {
+    float y = (load(i) - mean) * rstd;
+    if (gamma)
+      y *= float(gamma[i]);
+    if (beta)
+      y += float(beta[i]);
+    orow[i] = T(y);
+  }
+}
+
+template <typename T, int VPL>
+void launchWave(const T *x, const T *res, const T *gamma, const T *beta, T *out,
+                int64_t rows, int hidden, float eps, hipStream_t s) {
+  const int rowsPerBlock = 256 / kWave;
+  dim3 grid((unsigned)((rows + rowsPerBlock - 1) / rowsPerBlock)), block(256);
+  const bool affine = gamma || beta;
+  if (res) {
+    if (affine)
+      layernormWaveKernel<T, VPL, true, true>
+          <<<grid, block, 0, s>>>(x, res, gamma, beta, out, rows, hidden, eps);
+    else
+      layernormWaveKernel<T, VPL, true, false>
+          <<<grid, block, 0, s>>>(x, res, gamma, beta, out, rows, hidden, eps);
+  } else {
+    if (affine)
+      layernormWaveKernel<T, VPL, false, true>
+          <<<grid, block, 0, s>>>(x, res, gamma, beta, out, rows, hidden, eps);
+    else
+      layernormWaveKernel<T, VPL, false, false>
+          <<<grid, block, 0, s>>>(x, res, gamma, beta, out, rows, hidden, eps);
+  }
+}
+
+inline bool aligned16(const void *p) {
+  return (reinterpret_cast<uintptr_t>(p) & 15) == 0;
+}
+
+} // namespace
+
+template <typename T>
+Status launchLayernorm(const T *x, const T *res, const T *gamma, const T *beta,
+                       T *out, int64_t rows, int64_t hidden, float eps,
+                       hipStream_t s) {
+  if (rows == 0 || hidden == 0)
+    return Status::kSuccess;
+  HOM_CHECK_RET(rows < (int64_t(1) << 31), Status::kInvalidArgument,
+                "layernorm: too many rows (%lld)", (long long)rows);
+  constexpr int N = Vec16<T>::kN;
+  const bool vecOk = hidden % N == 0 && aligned16(x) && aligned16(out) &&
+                     (!res || aligned16(res)) && (!gamma || aligned16(gamma)) &&
+                     (!beta || aligned16(beta));
+  const int64_t nvec = hidden / N;
+  if (vecOk && nvec <= kWave * 8) {
+    const int h = int(hidden);
+    if (nvec <= kWave)
+      launchWave<T, 1>(x, res, gamma, beta, out, rows, h, eps, s);
+    else if (nvec <= kWave * 2)
+      launchWave<T, 2>(x, res, gamma, beta, out, rows, h, eps, s);
+    else if (nvec <= kWave * 4)
+      launchWave<T, 4>(x, res, gamma, beta, out, rows, h, eps, s);
+    else
+      launchWave<T, 8>(x, res, gamma, beta, out, rows, h, eps, s);
+  } else {
+    layernormBlockKernel<T><<<dim3((unsigned)rows), dim3(256), 0, s>>>(
+        x, res, gamma, beta, out, rows, hidden, eps);
+  }
+  HOM_HIP_RET(hipGetLastError(), Status::kInternal);
+  return Status::kSuccess;
+}
+
+template Status launchLayernorm<_Float16>(const _Float16 *, const _Float16 *,
+                                          const _Float16 *, const _Float16 *,
+                                          _Float16 *, int64_t, int64_t, float,
+                                          hipStream_t);
+template Status launchLayernorm<float>(const float *, const float *,
+                                       const float *, const float *, float *,
+                                       int64_t, int64_t, float, hipStream_t);
+
+} // namespace hom

@@ -1,0 +1,792 @@
+#include "runners.h"
+
+#include <cerrno>
+#include <cmath>
+#include <cstring>
+#include <fstream>
+#include <sstream>
+#include <string>
+
+namespace hom {
+
+namespace {
+
+Epilogue epilogueFor(int64_t activation, bool nvtePath) {
+  if (activation == 2)
+    return Epilogue::kGeluTanh;
+  if (activation == 1)
+    return nvtePath ? Epilogue::kGeluTanh : Epilogue::kGeluErf;
+  return Epilogue::kLinear;
+}
+
+// Shape rules of GemmOperationRunner::construct_arguments
+// (include/NVGPUKernels/GemmRunner.h:244-287), with two relaxations: C may be
+// broadcast over the batch and/or row dimension (bias row / per-batch matrix),
+// as the CPU matmulAddF32 allows, and C is not inspected when beta == 0.
+struct GemmShapes {
+  int64_t batch, Mp, N, K;
+};
+
+Status checkGemmOperands(const View<_Float16> &A, const View<_Float16> &B,
+                         const View<_Float16> &C, const View<_Float16> &D,
+                         bool bIsNK, float beta, GemmShapes *out,
+                         GemmProblem *pr) {
+  HOM_CHECK_RET(A.rank == 3 && B.rank == 3 && C.rank == 3 && D.rank == 3,
+                Status::kInvalidArgument,
+                "gemm: all operands must have rank 3 (got %lld %lld %lld %lld)",
+                (long long)A.rank, (long long)B.rank, (long long)C.rank,
+                (long long)D.rank);
+  HOM_CHECK_RET(A.sizes && B.sizes && C.sizes && D.sizes,
+                Status::kInvalidArgument, "gemm: null descriptor");
+  const int64_t batch = A.sizes[0], Mp = A.sizes[1], K = A.sizes[2];
+  const int64_t bK = bIsNK ? B.sizes[2] : B.sizes[1];
+  const int64_t N = bIsNK ? B.sizes[1] : B.sizes[2];
+  HOM_CHECK_RET(K == bK, Status::kInvalidArgument,
+                "gemm: K mismatch, A is [..,%lld] but B contracts over %lld",
+                (long long)K, (long long)bK);
+  HOM_CHECK_RET(B.sizes[0] == 1 || B.sizes[0] == batch || batch == 1,
+                Status::kInvalidArgument,
+                "gemm: B batch %lld incompatible with A batch %lld",
+                (long long)B.sizes[0], (long long)batch);
+  HOM_CHECK_RET(D.sizes[0] == batch && D.sizes[1] == Mp && D.sizes[2] == N,
+                Status::kInvalidArgument,
+                "gemm: D is [%lld,%lld,%lld], expected [%lld,%lld,%lld]",
+                (long long)D.sizes[0], (long long)D.sizes[1],
+                (long long)D.sizes[2], (long long)batch, (long long)Mp,
+                (long long)N);
+  HOM_CHECK_RET(A.contiguous() && B.contiguous() && D.contiguous(),
+                Status::kInvalidArgument,
+                "gemm: operands must be contiguous row-major");
+  pr->ldc = 0;
+  pr->cRowPeriod = 1;
+  pr->C = nullptr;
+  if (beta != 0.f) {
+    HOM_CHECK_RET(C.sizes[2] == N, Status::kInvalidArgument,
+                  "gemm: C has %lld columns, expected %lld",
+                  (long long)C.sizes[2], (long long)N);
+    HOM_CHECK_RET((C.sizes[0] == batch || C.sizes[0] == 1) &&
+                      (C.sizes[1] == Mp || C.sizes[1] == 1),
+                  Status::kInvalidArgument,
+                  "gemm: C is [%lld,%lld,%lld], not broadcastable to "
+                  "[%lld,%lld,%lld]",
+                  (long long)C.sizes[0], (long long)C.sizes[1],
+                  (long long)C.sizes[2], (long long)batch, (long long)Mp,
+                  (long long)N);
+    HOM_CHECK_RET(C.contiguous(), Status::kInvalidArgument,
+                  "gemm: C must be contiguous row-major");
+    HOM_CHECK_RET(C.data != nullptr, Status::kInvalidArgument,
+                  "gemm: beta != 0 with a null C");
+    pr->C = C.data;
+    const bool rowsFull = C.sizes[1] == Mp;
+    const bool batchFull = C.sizes[0] == batch;
+    pr->ldc = N;
+    if (rowsFull && batchFull) {
+      pr->cRowPeriod = batch * Mp; // a full [b, M', N] source
+    } else if (rowsFull) {
+      pr->cRowPeriod = Mp; // one [M', N] matrix shared by every batch
+    } else {
+      // a single bias row; one row per batch cannot be expressed as a period
+      HOM_CHECK_RET(C.sizes[0] == 1 || batch == 1, Status::kInvalidArgument,
+                    "gemm: C broadcast over rows but not over batch is not "
+                    "supported");
+      pr->cRowPeriod = 1;
+    }
+  }
+  pr->A = A.data;
+  pr->B = B.data;
+  pr->D = D.data;
+  pr->M = batch * Mp;
+  pr->N = N;
+  pr->K = K;
+  pr->lda = K;
+  pr->ldb = bIsNK ? K : N;
+  pr->ldd = N;
+  pr->bIsNK = bIsNK;
+  if (pr->cRowPeriod < 1)
+    pr->cRowPeriod = 1;
+  out->batch = batch;
+  out->Mp = Mp;
+  out->N = N;
+  out->K = K;
+  return Status::kSuccess;
+}
+
+int findKernel(int tileM, int tileN, int tileK, Epilogue epi, int alignment) {
+  for (int i = 0; i < gemmKernelCount(); i++) {
+    const GemmKernelInfo &k = gemmKernelInfo(i);
+    if (k.tileM == tileM && k.tileN == tileN && k.tileK == tileK &&
+        k.epilogue == epi && k.alignment == alignment)
+      return i;
+  }
+  return -1;
+}
+
+struct TunedEntry {
+  int64_t M, N, K;
+  int activation; // 0 linear, 1 gelu erf, 2 gelu tanh
+  const char *kernel;
+  int splitK;
+};
+
+// Produced on an MI355X by the autotuner (hands-on-mlir_amd/tune_gemm.py) for
+// the GEMM shapes of BERT-base and BERT-large; replaces the role of the
+// CUTLASS manifest generator's per-architecture tile lists
+// (python/gemm_generator.py:237-278).
+const TunedEntry kTuned[] = {
+#include "gemm_tuned_table.inc"
+    {0, 0, 0, 0, nullptr, 0}};
+
+int alignmentClass(const GemmProblem &p) {
+  auto a16 = [](const void *q) {
+    return (reinterpret_cast<uintptr_t>(q) & 15) == 0;
+  };
+  const bool ok = p.N % 8 == 0 && p.K % 8 == 0 && a16(p.A) && a16(p.B) &&
+                  a16(p.D) && (p.C == nullptr || a16(p.C));
+  return ok ? 8 : 1;
+}
+
+} // namespace
+
+bool selectGemm(int64_t M, int64_t N, int64_t K, int64_t activation,
+                int64_t *idx, int32_t *splitK) {
+  const Epilogue epi = epilogueFor(activation, false);
+  if (N % 8 == 0 && K % 8 == 0) {
+    for (const TunedEntry *t = kTuned; t->kernel; t++) {
+      if (t->M == M && t->N == N && t->K == K && t->activation == activation) {
+        for (int i = 0; i < gemmKernelCount(); i++) {
+          if (strcmp(gemmKernelInfo(i).name, t->kernel) == 0) {
+            *idx = i;
+            *splitK = t->splitK;
+            return true;
+          }
+        }
+      }
+    }
+  }
+  // Heuristic: estimate each tile's time as (rounds of workgroups over the
+  // chip) x (tile work / tile efficiency) and take the cheapest; small output
+  // grids get split-K until the chip is covered.
+  const int align = (N % 8 == 0 && K % 8 == 0) ? 8 : 1;
+  const int cus = deviceInfo().computeUnits > 0 ? deviceInfo().computeUnits : 256;
+  double bestCost = 1e300;
+  int best = -1, bestSplit = 1;
+  for (int i = 0; i < gemmKernelCount(); i++) {
+    const GemmKernelInfo &k = gemmKernelInfo(i);
+    if (k.epilogue != epi || k.alignment != align)
+      continue;
+    const int64_t tiles = ((M + k.tileM - 1) / k.tileM) *
+                          ((N + k.tileN - 1) / k.tileN);
+    const int kTiles = int((K + k.tileK - 1) / k.tileK);
+    // Relative MFMA efficiency of a tile: larger tiles reuse LDS data more.
+    const double eff =
+        double(k.tileM) * k.tileN / (double(k.tileM + k.tileN) * 64.0);
+    const int maxSplit = std::max(1, std::min(16, int(K / 128)));
+    for (int s = 1; s <= maxSplit; s++) {
+      if (s > kTiles)
+        break;
+      const double slots = double(cus) * 2.0;
+      const double rounds = std::ceil(double(tiles) * s / slots);
+      const double work = double(k.tileM) * k.tileN * (double(K) / s);
+      double cost = rounds * (work / eff + 2.0e5);
+      if (s > 1)
+        cost += double(k.tileM) * k.tileN * s * 8.0 + 4.0e5; // reduction pass
+      if (cost < bestCost) {
+        bestCost = cost;
+        best = i;
+        bestSplit = s;
+      }
+    }
+  }
+  if (best < 0) {
+    best = findKernel(64, 64, 32, epi, 1);
+    bestSplit = 1;
+  }
+  *idx = best;
+  *splitK = bestSplit;
+  return false;
+}
+
+Status runGemmManifest(int64_t rankA, void *dstA, int64_t rankB, void *dstB,
+                       int64_t rankC, void *dstC, int64_t rankD, void *dstD,
+                       int64_t activation, float alpha, float beta,
+                       int32_t gemmNum, int32_t splitK) {
+  View<_Float16> A(rankA, dstA), B(rankB, dstB), C(rankC, dstC), D(rankD, dstD);
+  GemmProblem pr{};
+  GemmShapes sh{};
+  Status st = checkGemmOperands(A, B, C, D, false, beta, &sh, &pr);
+  if (st != Status::kSuccess)
+    return st;
+  pr.alpha = alpha;
+  pr.beta = beta;
+  int idx;
+  if (gemmNum >= 1) {
+    HOM_CHECK_RET(gemmNum <= gemmKernelCount(), Status::kInvalidArgument,
+                  "gemm: kernel number %d outside the manifest (1..%d)",
+                  gemmNum, gemmKernelCount());
+    idx = gemmNum - 1;
+    HOM_CHECK_RET(splitK >= 1, Status::kInvalidArgument,
+                  "gemm: split-K factor must be >= 1 (got %d)", splitK);
+    pr.splitK = splitK;
+  } else {
+    // The reference indexes manifest[-1] here (undefined); this library
+    // treats 0 as "choose for me" using the activation argument.
+    HOM_CHECK_RET(gemmNum == 0, Status::kInvalidArgument,
+                  "gemm: negative kernel number %d", gemmNum);
+    int64_t sel;
+    int32_t sk;
+    selectGemm(pr.M, pr.N, pr.K, activation, &sel, &sk);
+    idx = int(sel);
+    pr.splitK = sk;
+    if (gemmKernelInfo(idx).alignment == 8 && alignmentClass(pr) != 8) {
+      idx = findKernel(64, 64, 32, gemmKernelInfo(idx).epilogue, 1);
+      pr.splitK = 1;
+    }
+  }
+  return launchGemm(idx, pr, stream());
+}
+
+Status runGemmNvte(int64_t rankA, void *dstA, bool transa, int64_t rankB,
+                   void *dstB, bool transb, int64_t rankC, void *dstC,
+                   int64_t rankD, void *dstD, int64_t activation, float alpha,
+                   float beta) {
+  // Preconditions of GemmNVTERunner::construct_tensors (GemmRunner.h:342-381).
+  HOM_CHECK_RET(transa == false, Status::kInvalidArgument,
+                "nvte gemm: transa must be false");
+  HOM_CHECK_RET(transb == true, Status::kInvalidArgument,
+                "nvte gemm: transb must be true (B is [1, N, K])");
+  HOM_CHECK_RET(alpha == 1.0f, Status::kInvalidArgument,
+                "nvte gemm: alpha must be 1 (got %g)", double(alpha));
+  HOM_CHECK_RET(beta == 0.0f || beta == 1.0f, Status::kInvalidArgument,
+                "nvte gemm: beta must be 0 or 1 (got %g)", double(beta));
+  HOM_CHECK_RET(activation >= 0 && activation <= 2, Status::kInvalidArgument,
+                "nvte gemm: unknown activation %lld", (long long)activation);
+  View<_Float16> A(rankA, dstA), B(rankB, dstB), C(rankC, dstC), D(rankD, dstD);
+  GemmProblem pr{};
+  GemmShapes sh{};
+  Status st = checkGemmOperands(A, B, C, D, true, beta, &sh, &pr);
+  if (st != Status::kSuccess)
+    return st;
+  HOM_CHECK_RET(B.sizes[0] == 1, Status::kInvalidArgument,
+                "nvte gemm: B batch must be 1");
+  if (beta != 0.f) {
+    HOM_CHECK_RET(C.data == D.data, Status::kInvalidArgument,
+                  "nvte gemm: beta == 1 accumulates in place, C must alias D");
+  }
+  pr.alpha = alpha;
+  pr.beta = beta;
+  int64_t sel;
+  int32_t sk;
+  const Epilogue epi = epilogueFor(activation, true);
+  selectGemm(pr.M, pr.N, pr.K, epi == Epilogue::kGeluTanh ? 2 : activation,
+             &sel, &sk);
+  int idx = int(sel);
+  pr.splitK = sk;
+  if (gemmKernelInfo(idx).alignment == 8 && alignmentClass(pr) != 8) {
+    idx = findKernel(64, 64, 32, epi, 1);
+    pr.splitK = 1;
+  }
+  return launchGemm(idx, pr, stream());
+}
+
+Status runGemmWithVarMean(int64_t rankA, void *dstA, int64_t rankB, void *dstB,
+                          int64_t rankC, void *dstC, int64_t rankD, void *dstD,
+                          int64_t rankVar, void *dstVar, int64_t rankMean,
+                          void *dstMean, float alpha, float beta,
+                          int64_t activation, float eps) {
+  (void)activation; // linear epilogue only, as in the reference instance
+  View<_Float16> D(rankD, dstD), Var(rankVar, dstVar), Mean(rankMean, dstMean);
+  Status st = runGemmManifest(rankA, dstA, rankB, dstB, rankC, dstC, rankD,
+                              dstD, 0, alpha, beta, 0, 1);
+  if (st != Status::kSuccess)
+    return st;
+  const int64_t rows = D.sizes[0] * D.sizes[1], n = D.sizes[2];
+  HOM_CHECK_RET(Var.sizes && Mean.sizes && Var.numel() >= rows &&
+                    Mean.numel() >= rows,
+                Status::kInvalidArgument,
+                "gemm+stats: Var/Mean need one element per output row (%lld)",
+                (long long)rows);
+  return launchRowStatsF16(D.data, Var.data, Mean.data, rows, n, eps, stream());
+}
+
+Status runLayernormGemm(int64_t rankA, void *dstA, int64_t rankB, void *dstB,
+                        int64_t rankC, void *dstC, int64_t rankD, void *dstD,
+                        int64_t rankVar, void *dstVar, int64_t rankMean,
+                        void *dstMean, float alpha, float beta,
+                        int64_t activation) {
+  (void)activation;
+  View<_Float16> A(rankA, dstA), Var(rankVar, dstVar), Mean(rankMean, dstMean);
+  HOM_CHECK_RET(A.rank == 3 && A.sizes && A.contiguous(),
+                Status::kInvalidArgument,
+                "layernorm-gemm: A must be a contiguous rank-3 tensor");
+  const int64_t rows = A.sizes[0] * A.sizes[1], k = A.sizes[2];
+  HOM_CHECK_RET(Var.sizes && Mean.sizes && Var.numel() >= rows &&
+                    Mean.numel() >= rows,
+                Status::kInvalidArgument,
+                "layernorm-gemm: Var/Mean need one element per row (%lld)",
+                (long long)rows);
+  _Float16 *tmp = static_cast<_Float16 *>(
+      scratch(kTemp, size_t(rows) * k * sizeof(_Float16), false));
+  if (!tmp && rows * k > 0)
+    return Status::kInternal;
+  Status st = launchApplyRowStatsF16(A.data, Var.data, Mean.data, tmp, rows, k,
+                                     stream());
+  if (st != Status::kSuccess)
+    return st;
+  // Same descriptor as A, pointing at the normalised copy.
+  HomStridedMemRef3 normA;
+  memcpy(&normA, dstA, sizeof(normA));
+  normA.basePtr = normA.data = tmp;
+  return runGemmManifest(3, &normA, rankB, dstB, rankC, dstC, rankD, dstD, 0,
+                         alpha, beta, 0, 1);
+}
+
+// ---------------------------------------------------------------- profiler --
+GemmProfiler::GemmProfiler(int64_t M, int64_t N, int64_t K, int64_t activation,
+                           float alpha, float beta)
+    : M_(M), N_(N), K_(K), activation_(activation), alpha_(alpha), beta_(beta) {
+  if (hipEventCreate(&start_) != hipSuccess ||
+      hipEventCreate(&stop_) != hipSuccess)
+    recordError(__FILE__, __LINE__, "profiler: cannot create HIP events");
+}
+
+GemmProfiler::~GemmProfiler() {
+  if (start_)
+    (void)hipEventDestroy(start_);
+  if (stop_)
+    (void)hipEventDestroy(stop_);
+  for (Buffer *b : {&a_, &b_, &c_})
+    if (b->data)
+      (void)hipFree(b->data);
+}
+
+bool GemmProfiler::ensure(Buffer &b, int64_t elems) {
+  if (elems <= b.capacity)
+    return true;
+  if (b.data)
+    (void)hipFree(b.data);
+  b.data = nullptr;
+  b.capacity = 0;
+  void *p = nullptr;
+  if (hipMalloc(&p, size_t(elems) * sizeof(_Float16)) != hipSuccess) {
+    recordError(__FILE__, __LINE__, "profiler: hipMalloc of %lld halves failed",
+                (long long)elems);
+    return false;
+  }
+  // Zeros: timing does not depend on the values, and NaN patterns are avoided.
+  (void)hipMemset(p, 0, size_t(elems) * sizeof(_Float16));
+  b.data = static_cast<_Float16 *>(p);
+  b.capacity = elems;
+  return true;
+}
+
+// Protocol of GemmProfiler::profileHelper (lib/NVGPUKernels/GemmProfiler.cu:
+// 81-120): 10 warm-up launches, then batches of 100 between two events until
+// 500 ms have been spent or the kernel is 1.2x slower than the best so far.
+float GemmProfiler::timeKernel(int idx, int splitK, float previousBest) {
+  GemmProblem pr{};
+  pr.A = a_.data;
+  pr.B = b_.data;
+  pr.C = beta_ != 0.f ? c_.data : nullptr;
+  pr.D = c_.data;
+  pr.M = M_;
+  pr.N = N_;
+  pr.K = K_;
+  pr.lda = K_;
+  pr.ldb = N_;
+  pr.ldc = N_;
+  pr.ldd = N_;
+  pr.cRowPeriod = M_;
+  pr.alpha = alpha_;
+  pr.beta = beta_;
+  pr.bIsNK = false;
+  pr.splitK = splitK;
+  hipStream_t s = stream();
+  if (hipStreamSynchronize(s) != hipSuccess)
+    return INFINITY;
+  for (int i = 0; i < 10; i++)
+    if (launchGemm(idx, pr, s) != Status::kSuccess)
+      return INFINITY;
+  float total = 0.f;
+  int64_t iters = 0;
+  while (total < 500.f) {
+    float batch = 0.f;
+    (void)hipEventRecord(start_, s);
+    for (int i = 0; i < 100; i++)
+      (void)launchGemm(idx, pr, s);
+    (void)hipEventRecord(stop_, s);
+    if (hipEventSynchronize(stop_) != hipSuccess)
+      return INFINITY;
+    (void)hipEventElapsedTime(&batch, start_, stop_);
+    total += batch;
+    iters += 100;
+    if (total / float(iters) / 1.2f > previousBest)
+      break;
+  }
+  return total / float(iters);
+}
+
+std::tuple<int64_t, int32_t> GemmProfiler::profile() {
+  const auto key = std::make_tuple(M_, N_, K_, activation_);
+  auto it = cache_.find(key);
+  if (it != cache_.end()) {
+    bestTimeMs_ = std::get<2>(it->second);
+    fprintf(stderr, "Cache hit, Idx = %lld, split k factor = %d\n",
+            (long long)std::get<0>(it->second), std::get<1>(it->second));
+    return {std::get<0>(it->second), std::get<1>(it->second)};
+  }
+  if (!ensure(a_, M_ * K_) || !ensure(b_, K_ * N_) || !ensure(c_, M_ * N_))
+    return {-1, 1};
+  const Epilogue epi = epilogueFor(activation_, false);
+  // Alignment class: largest of {8, 1} dividing N and K (the reference walks
+  // {8,4,2,1} over M, N, K: lib/NVGPUKernels/GemmProfiler.cu:170-180; row
+  // count does not constrain these kernels).
+  const int align = (N_ % 8 == 0 && K_ % 8 == 0) ? 8 : 1;
+  const int maxSplit = std::max(1, std::min<int>(16, int(K_ / 128)));
+  const int cus = deviceInfo().computeUnits > 0 ? deviceInfo().computeUnits : 256;
+
+  int64_t bestIdx = -1;
+  int32_t bestSplit = 1;
+  float bestTime = INFINITY;
+  for (int idx = 0; idx < gemmKernelCount(); idx++) {
+    const GemmKernelInfo &k = gemmKernelInfo(idx);
+    if (k.epilogue != epi || k.alignment > align)
+      continue;
+    if (k.alignment < align && align == 8)
+      continue; // the scalar-access kernels never win on aligned problems
+    const int64_t tiles = ((M_ + k.tileM - 1) / k.tileM) *
+                          ((N_ + k.tileN - 1) / k.tileN);
+    for (int s = 1; s <= maxSplit; s++) {
+      // Slicing K further once the grid already covers the chip many times
+      // only adds reduction traffic; skip those candidates.
+      if (s > 1 && tiles * (s - 1) >= int64_t(cus) * 4)
+        break;
+      const float t = timeKernel(idx, s, bestTime);
+      if (t < bestTime) {
+        bestTime = t;
+        bestIdx = idx;
+        bestSplit = s;
+      }
+    }
+  }
+  bestTimeMs_ = bestTime;
+  fprintf(stderr,
+          "Profile for %lld %lld %lld act: %lld done. Best kernel %s, best "
+          "split k factor %d, best time %g ms (%.1f TFLOP/s).\n",
+          (long long)M_, (long long)N_, (long long)K_, (long long)activation_,
+          bestIdx >= 0 ? gemmKernelInfo(int(bestIdx)).name : "none", bestSplit,
+          double(bestTime),
+          2.0 * double(M_) * double(N_) * double(K_) / (double(bestTime) * 1e9));
+  cache_[key] = std::make_tuple(bestIdx, bestSplit, bestTime);
+  return {bestIdx, bestSplit};
+}
+
+std::tuple<int64_t, int32_t> GemmProfiler::profile(int64_t M, int64_t N,
+                                                   int64_t K,
+                                                   int64_t activation,
+                                                   float alpha, float beta) {
+  M_ = M;
+  N_ = N;
+  K_ = K;
+  activation_ = activation;
+  alpha_ = alpha;
+  beta_ = beta;
+  return profile();
+}
+
+// ------------------------------------------------------------- layer norm --
+template <typename T>
+Status runLayernorm(int64_t rankA, void *dstA, float eps) {
+  View<T> A(rankA, dstA);
+  // LayernormRunner::construct_tensors (Layernorm.h:619-624)
+  HOM_CHECK_RET((A.rank == 3 || A.rank == 2) && A.sizes,
+                Status::kInvalidArgument,
+                "layernorm: rank must be 2 or 3 (got %lld)", (long long)A.rank);
+  HOM_CHECK_RET(A.contiguous(), Status::kInvalidArgument,
+                "layernorm: tensor must be contiguous row-major");
+  const int64_t rows = A.rank == 3 ? A.sizes[0] * A.sizes[1] : A.sizes[0];
+  const int64_t hidden = A.rank == 3 ? A.sizes[2] : A.sizes[1];
+  return launchLayernorm<T>(A.data, nullptr, nullptr, nullptr, A.data, rows,
+                            hidden, eps, stream());
+}
+template Status runLayernorm<_Float16>(int64_t, void *, float);
+template Status runLayernorm<float>(int64_t, void *, float);
+
+Status runAddLayernormF16(int64_t rankX, void *dstX, int64_t rankRes,
+                          void *dstRes, int64_t rankGamma, void *dstGamma,
+                          int64_t rankBeta, void *dstBeta, int64_t rankOut,
+                          void *dstOut, float eps) {
+  View<_Float16> X(rankX, dstX), R(rankRes, dstRes), G(rankGamma, dstGamma),
+      Bt(rankBeta, dstBeta), O(rankOut, dstOut);
+  HOM_CHECK_RET((X.rank == 3 || X.rank == 2) && X.sizes && O.sizes &&
+                    O.rank == X.rank,
+                Status::kInvalidArgument,
+                "add+layernorm: X and Out must both have rank 2 or 3");
+  for (int64_t i = 0; i < X.rank; i++)
+    HOM_CHECK_RET(X.sizes[i] == O.sizes[i], Status::kInvalidArgument,
+                  "add+layernorm: Out shape differs from X in dim %lld",
+                  (long long)i);
+  HOM_CHECK_RET(X.contiguous() && O.contiguous(), Status::kInvalidArgument,
+                "add+layernorm: X and Out must be contiguous");
+  const int64_t rows = X.rank == 3 ? X.sizes[0] * X.sizes[1] : X.sizes[0];
+  const int64_t hidden = X.rank == 3 ? X.sizes[2] : X.sizes[1];
+  if (dstRes) {
+    HOM_CHECK_RET(R.rank == X.rank && R.contiguous(), Status::kInvalidArgument,
+                  "add+layernorm: Res must match X");
+    for (int64_t i = 0; i < X.rank; i++)
+      HOM_CHECK_RET(X.sizes[i] == R.sizes[i], Status::kInvalidArgument,
+                    "add+layernorm: Res shape differs from X in dim %lld",
+                    (long long)i);
+  }
+  if (dstGamma)
+    HOM_CHECK_RET(G.numel() == hidden && G.contiguous(),
+                  Status::kInvalidArgument,
+                  "add+layernorm: Gamma must hold %lld values",
+                  (long long)hidden);
+  if (dstBeta)
+    HOM_CHECK_RET(Bt.numel() == hidden && Bt.contiguous(),
+                  Status::kInvalidArgument,
+                  "add+layernorm: Beta must hold %lld values",
+                  (long long)hidden);
+  return launchLayernorm<_Float16>(X.data, dstRes ? R.data : nullptr,
+                                   dstGamma ? G.data : nullptr,
+                                   dstBeta ? Bt.data : nullptr, O.data, rows,
+                                   hidden, eps, stream());
+}
+
+// --------------------------------------------------------------- attention --
+Status runBertAttentionF16(int64_t rankA, void *dstA, int64_t rankSeqlen,
+                           void *dstSeqlen, int64_t rankOut, void *dstOut,
+                           float scale, int64_t headNum) {
+  View<_Float16> A(rankA, dstA), Out(rankOut, dstOut);
+  View<int32_t> Seq(rankSeqlen, dstSeqlen);
+  // BertAttentionRunner::construct_tensors (BertAttentionRunner.h:61-73)
+  HOM_CHECK_RET(A.rank == 3 && A.sizes, Status::kInvalidArgument,
+                "attention: QKV must have rank 3 (got %lld)",
+                (long long)A.rank);
+  HOM_CHECK_RET(headNum > 0 && A.sizes[2] % (headNum * 3) == 0,
+                Status::kInvalidArgument,
+                "attention: last dim %lld is not a multiple of 3 * heads (%lld)",
+                (long long)A.sizes[2], (long long)headNum);
+  HOM_CHECK_RET(Out.rank == 3 && Out.sizes, Status::kInvalidArgument,
+                "attention: Out must have rank 3");
+  HOM_CHECK_RET(Out.sizes[0] == A.sizes[0] && Out.sizes[1] == A.sizes[1] &&
+                    Out.sizes[2] * 3 == A.sizes[2],
+                Status::kInvalidArgument,
+                "attention: Out is [%lld,%lld,%lld] for QKV [%lld,%lld,%lld]",
+                (long long)Out.sizes[0], (long long)Out.sizes[1],
+                (long long)Out.sizes[2], (long long)A.sizes[0],
+                (long long)A.sizes[1], (long long)A.sizes[2]);
+  const int64_t bs = A.sizes[0], seq = A.sizes[1];
+  const int64_t headDim = A.sizes[2] / headNum / 3;
+  HOM_CHECK_RET(Seq.rank == 1 && Seq.sizes && Seq.sizes[0] == bs + 1,
+                Status::kInvalidArgument,
+                "attention: cu_seqlens must be int32[%lld]", (long long)bs + 1);
+  HOM_CHECK_RET(A.contiguous() && Out.contiguous(), Status::kInvalidArgument,
+                "attention: tensors must be contiguous");
+  return launchBertAttentionF16(A.data, Seq.data, Out.data, bs, seq, headNum,
+                                headDim, scale, stream());
+}
+
+// ------------------------------------------------------------- elementwise --
+template <typename T>
+Status runElementwise(BinOp op, int64_t rankA, void *dstA, int64_t rankB,
+                      void *dstB, int64_t rankOut, void *dstOut) {
+  View<T> A(rankA, dstA), B(rankB, dstB), Out(rankOut, dstOut);
+  // ElementwiseRunner::run (ElementwiseRunner.h:132-138)
+  HOM_CHECK_RET(A.rank == B.rank && A.rank == Out.rank,
+                Status::kInvalidArgument,
+                "elementwise: ranks differ (%lld, %lld, %lld)",
+                (long long)A.rank, (long long)B.rank, (long long)Out.rank);
+  HOM_CHECK_RET(A.rank >= 0 && A.rank <= kMaxRank, Status::kInvalidArgument,
+                "elementwise: rank %lld not supported (max %d)",
+                (long long)A.rank, kMaxRank);
+  HOM_CHECK_RET(A.rank == 0 || (A.sizes && B.sizes && Out.sizes),
+                Status::kInvalidArgument, "elementwise: null descriptor");
+  BroadcastDesc d{};
+  d.rank = int(A.rank);
+  for (int64_t i = 0; i < A.rank; i++) {
+    HOM_CHECK_RET(A.sizes[i] == B.sizes[i] || B.sizes[i] == 1,
+                  Status::kInvalidArgument,
+                  "elementwise: only B can broadcast (dim %lld: A %lld, B %lld)",
+                  (long long)i, (long long)A.sizes[i], (long long)B.sizes[i]);
+    HOM_CHECK_RET(A.sizes[i] == Out.sizes[i], Status::kInvalidArgument,
+                  "elementwise: Out differs from A in dim %lld", (long long)i);
+  }
+  HOM_CHECK_RET(A.contiguous() && Out.contiguous(), Status::kInvalidArgument,
+                "elementwise: A and Out must be contiguous row-major");
+  int64_t stride = 1;
+  for (int64_t i = A.rank - 1; i >= 0; i--) {
+    d.outSize[i] = A.sizes[i];
+    d.outStride[i] = stride;
+    stride *= A.sizes[i];
+    d.bSize[i] = B.sizes[i];
+    d.bStride[i] = B.sizes[i] == 1 ? 0 : B.strides[i];
+  }
+  return launchElementwise<T>(op, A.data, B.data, Out.data, A.numel(), d,
+                              stream());
+}
+template Status runElementwise<_Float16>(BinOp, int64_t, void *, int64_t,
+                                         void *, int64_t, void *);
+template Status runElementwise<float>(BinOp, int64_t, void *, int64_t, void *,
+                                      int64_t, void *);
+
+template <typename T>
+Status runGather(int64_t rankIdx, void *desIdx, int64_t rankValue,
+                 void *desValue, int64_t rankOut, void *desOut) {
+  View<int64_t> I(rankIdx, desIdx);
+  View<T> V(rankValue, desValue), O(rankOut, desOut);
+  // GatherRunner::run (GatherRunner.h:52-60)
+  HOM_CHECK_RET(V.rank == 3 && V.sizes && V.sizes[0] == 1,
+                Status::kInvalidArgument,
+                "gather: value must be [1, V, H] (rank %lld)",
+                (long long)V.rank);
+  HOM_CHECK_RET(I.rank == 2 && I.sizes && O.sizes && O.rank == 3,
+                Status::kInvalidArgument,
+                "gather: indices must have rank 2 and out rank 3");
+  HOM_CHECK_RET(O.sizes[2] == V.sizes[2] && I.sizes[0] == O.sizes[0] &&
+                    I.sizes[1] == O.sizes[1],
+                Status::kInvalidArgument, "gather: shape mismatch");
+  HOM_CHECK_RET(I.contiguous() && V.contiguous() && O.contiguous(),
+                Status::kInvalidArgument, "gather: tensors must be contiguous");
+  return launchGather<T>(I.data, V.data, O.data, I.sizes[0] * I.sizes[1],
+                         V.sizes[1], V.sizes[2], stream());
+}
+template Status runGather<_Float16>(int64_t, void *, int64_t, void *, int64_t,
+                                    void *);
+template Status runGather<float>(int64_t, void *, int64_t, void *, int64_t,
+                                 void *);
+
+template <typename InT>
+Status runCuSeqLen(int64_t rankIn, void *desIn, int64_t rankOut, void *desOut) {
+  View<InT> In(rankIn, desIn);
+  View<int32_t> Out(rankOut, desOut);
+  // CuSeqLenRunner::run (CuSeqLen.h:55-57)
+  HOM_CHECK_RET(In.rank == 2 && In.sizes, Status::kInvalidArgument,
+                "cu_seqlens: mask must have rank 2 (got %lld)",
+                (long long)In.rank);
+  HOM_CHECK_RET(Out.rank == 1 && Out.sizes, Status::kInvalidArgument,
+                "cu_seqlens: out must have rank 1");
+  HOM_CHECK_RET(In.sizes[0] + 1 == Out.sizes[0], Status::kInvalidArgument,
+                "cu_seqlens: out has %lld entries, expected %lld",
+                (long long)Out.sizes[0], (long long)In.sizes[0] + 1);
+  HOM_CHECK_RET(In.contiguous(), Status::kInvalidArgument,
+                "cu_seqlens: mask must be contiguous");
+  return launchCuSeqLen<InT>(In.data, Out.data, In.sizes[0], In.sizes[1],
+                             stream());
+}
+template Status runCuSeqLen<int64_t>(int64_t, void *, int64_t, void *);
+template Status runCuSeqLen<int32_t>(int64_t, void *, int64_t, void *);
+
+Status runGeluF16(int64_t rankA, void *dstA, int64_t rankOut, void *dstOut,
+                  int32_t form) {
+  View<_Float16> A(rankA, dstA), O(rankOut, dstOut);
+  HOM_CHECK_RET(A.sizes && O.sizes && A.rank == O.rank,
+                Status::kInvalidArgument, "gelu: rank mismatch");
+  HOM_CHECK_RET(A.numel() == O.numel() && A.contiguous() && O.contiguous(),
+                Status::kInvalidArgument,
+                "gelu: tensors must be contiguous and equally sized");
+  HOM_CHECK_RET(form == 0 || form == 1, Status::kInvalidArgument,
+                "gelu: form must be 0 (erf) or 1 (tanh)");
+  return launchGeluF16(A.data, O.data, A.numel(), form, stream());
+}
+
+// ------------------------------------------------------------------ memory --
+C_UnrankedMemRefType allocDevice(const std::vector<int64_t> &sizes,
+                                 size_t elemBytes) {
+  C_UnrankedMemRefType res{int64_t(sizes.size()), nullptr};
+  const size_t rank = sizes.size();
+  int64_t total = 1;
+  for (int64_t s : sizes) {
+    HOM_CHECK_RET(s >= 0, res, "alloc: negative extent %lld", (long long)s);
+    total *= s;
+  }
+  const size_t descBytes = sizeof(HomMemRefHeader) + 2 * rank * sizeof(int64_t);
+  void *desc = malloc(descBytes);
+  HOM_CHECK_RET(desc != nullptr, res, "alloc: out of host memory");
+  void *dev = nullptr;
+  if (total > 0) {
+    hipError_t e = hipMalloc(&dev, size_t(total) * elemBytes);
+    if (e != hipSuccess) {
+      free(desc);
+      recordError(__FILE__, __LINE__, "alloc: hipMalloc of %zu bytes failed: %s",
+                  size_t(total) * elemBytes, hipGetErrorString(e));
+      return res;
+    }
+  }
+  auto *h = static_cast<HomMemRefHeader *>(desc);
+  h->basePtr = dev;
+  h->data = dev;
+  h->offset = 0;
+  int64_t *sz = hom_memref_sizes(desc);
+  int64_t *st = hom_memref_strides(desc, int64_t(rank));
+  int64_t stride = 1;
+  for (size_t i = 0; i < rank; i++) {
+    sz[i] = sizes[i];
+    st[rank - i - 1] = stride;
+    stride *= sizes[rank - i - 1];
+  }
+  res.descriptor = desc;
+  return res;
+}
+
+// Text format written by the reference's weight serialiser
+// (lib/WeightsEngine/WeightsEngine.cpp:22-39) and read back by
+// allocConstantNVGPU* (HandsOnNVGPURunnerUtils.cu:224-298): first line the
+// three extents, then the values as decimal text.
+template <typename T> C_UnrankedMemRefType allocConstant(int32_t idx) {
+  C_UnrankedMemRefType res{3, nullptr};
+  const char *dir = getenv("HOM_CONSTANT_DIR");
+  std::string path = std::string(dir ? dir : ".") + "/" + std::to_string(idx) +
+                     ".txt";
+  FILE *f = fopen(path.c_str(), "rb");
+  HOM_CHECK_RET(f != nullptr, res, "constant %d: cannot open %s (%s)", idx,
+                path.c_str(), strerror(errno));
+  std::string text;
+  {
+    char buf[1 << 16];
+    size_t n;
+    while ((n = fread(buf, 1, sizeof(buf), f)) > 0)
+      text.append(buf, n);
+    fclose(f);
+  }
+  const size_t eol = text.find('\n');
+  std::vector<int64_t> dims;
+  {
+    std::stringstream ss(text.substr(0, eol));
+    int64_t v;
+    while (ss >> v)
+      dims.push_back(v);
+  }
+  HOM_CHECK_RET(dims.size() == 3, res,
+                "constant %d: header of %s has %zu extents, expected 3", idx,
+                path.c_str(), dims.size());
+  int64_t total = dims[0] * dims[1] * dims[2];
+  std::vector<T> host;
+  host.resize(size_t(total));
+  const char *p = eol == std::string::npos ? text.c_str() + text.size()
+                                           : text.c_str() + eol + 1;
+  for (int64_t i = 0; i < total; i++) {
+    char *end = nullptr;
+    const float v = strtof(p, &end);
+    HOM_CHECK_RET(end != p, res,
+                  "constant %d: %s holds %lld values, expected %lld", idx,
+                  path.c_str(), (long long)i, (long long)total);
+    host[size_t(i)] = T(v); // float -> half rounds to nearest even
+    p = end;
+  }
+  res = allocDevice(dims, sizeof(T));
+  if (!res.descriptor)
+    return res;
+  if (total > 0) {
+    hipError_t e = hipMemcpy(hom_memref_data(res.descriptor), host.data(),
+                             size_t(total) * sizeof(T), hipMemcpyHostToDevice);
+    if (e != hipSuccess)
+      recordError(__FILE__, __LINE__, "constant %d: upload failed: %s", idx,
+                  hipGetErrorString(e));
+  }
+  return res;
+}
+template C_UnrankedMemRefType allocConstant<_Float16>(int32_t);
+template C_UnrankedMemRefType allocConstant<float>(int32_t);
+
+} // namespace hom

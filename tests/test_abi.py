@@ -1,0 +1,171 @@
+"""CPU-side checks of the drop-in boundary: the library loads, exports every
+symbol the header declares, and rejects bad arguments before touching the GPU."""
+import ctypes
+import os
+import re
+import subprocess
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "hom_amdgpu_runner_utils.h")
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    names = set(re.findall(r"HOM_EXPORT\s+[\w\s\*]+?\b(\w+)\s*\(", text))
+    for op, sfx in re.findall(r"HOM_ELEMENTWISE_DECL\((\w+), (\w+)\)", text):
+        names.add(f"thrustElementwise{op}{sfx}")
+    names.discard("thrustElementwiseopsuffix")
+    return names
+
+
+def test_header_symbols_all_exported(rt):
+    lib = rt.load_runtime()
+    names = declared_symbols()
+    assert len(names) >= 45
+    for n in sorted(names):
+        assert hasattr(lib, n), f"{n} declared in the header but not exported"
+    # and the ctypes table covers exactly the header
+    assert names == set(rt.SIGNATURES), names ^ set(rt.SIGNATURES)
+
+
+def test_reference_symbol_names_present(rt):
+    """Names the compiler emits calls to (include/Conversions/Function/FunctionUtils.h:12-49)."""
+    lib = rt.load_runtime()
+    for n in ["cutlassGemmF16", "cutlassGemmF32", "nvteGemmF16", "nvteLayernormF16", "nvteLayernormF32",
+              "nvteBertAttentionF16", "nvteBertAttentionF32", "alloc3DMemRefNVGPUF16",
+              "alloc3DMemRefNVGPUF32", "alloc1DMemRefNVGPUI32", "allocConstantNVGPUF16",
+              "allocConstantNVGPUF32", "deallocNVGPUF16", "deallocNVGPUF32", "deallocNVGPUI32",
+              "thrustElementwiseAddF16", "thrustElementwiseSubF32", "thrustGatherF16",
+              "thrustCuSeqLenI64", "thrustCuSeqLenI32", "cutlassGemmWithVarMeanF16",
+              "cutlassLayernormGemmF16", "cutlassLayernormGemmF32", "printMemrefSizeF16"]:
+        assert hasattr(lib, n)
+
+
+def test_unranked_memref_is_16_byte_pod(rt):
+    assert ctypes.sizeof(rt.CUnrankedMemRef) == 16
+
+
+def test_manifest_is_well_formed(rt):
+    man = rt.manifest()
+    assert len(man) >= 9
+    names = [m[1] for m in man]
+    assert len(set(names)) == len(names)
+    lib = rt.load_runtime()
+    for idx, name, act, align in man:
+        # activation is derived from the name the way the reference's runner does
+        # (GemmRunner.h:200-206): "gelu" -> 1, "linear" -> 0
+        assert act == (1 if "gelu" in name else 0)
+        assert ("linear" in name) != ("gelu" in name)
+        assert align in (1, 8)
+        assert lib.homGemmManifestFind(name.encode()) == idx
+    assert lib.homGemmManifestFind(b"no_such_kernel") == -1
+    assert lib.homGemmManifestName(-1) == b"" and lib.homGemmManifestActivation(10**6) == -1
+    # every (epilogue) has an unaligned fallback
+    assert any(a == 1 and "linear" in n for _, n, _, a in man)
+
+
+def test_select_returns_compatible_kernel(rt):
+    lib = rt.load_runtime()
+    man = rt.manifest()
+    idx, sk = ctypes.c_int64(), ctypes.c_int32()
+    for (M, N, K, act) in [(1024, 2304, 768, 0), (1024, 3072, 768, 1), (1024, 3072, 768, 2),
+                           (1024, 768, 3072, 0), (64, 1024, 4096, 0), (7, 13, 5, 0), (16384, 4096, 1024, 1)]:
+        lib.homGemmSelect(M, N, K, act, ctypes.byref(idx), ctypes.byref(sk))
+        _, name, a, align = man[idx.value]
+        assert a == (1 if act else 0)
+        assert ("gelutanh" in name) == (act == 2)
+        assert sk.value >= 1 and sk.value <= max(1, min(16, K // 128))
+        if N % 8 or K % 8:
+            assert align == 1
+
+
+# ---- argument checking: runs without a GPU because every check precedes the
+# first HIP call.  Default mode aborts (reference: assert / exit(1)); mode 1
+# records the message instead.
+def _errors(rt, fn):
+    lib = rt.load_runtime()
+    lib.homSetErrorMode(1)
+    try:
+        lib.homGetLastError()
+        fn(lib)
+        return lib.homGetLastError().decode()
+    finally:
+        lib.homSetErrorMode(0)
+
+
+def test_gemm_argument_checks(rt):
+    M = rt.MemRef
+    a, b, d = M(256, [1, 16, 32]), M(256, [1, 32, 8]), M(256, [1, 16, 8])
+
+    def call(A, B, C, D, num=1, sk=1, beta=0.0):
+        return lambda lib: lib.cutlassGemmF16(*A.args(), False, *B.args(), False, *C.args(), *D.args(),
+                                              0, 1.0, beta, num, sk)
+    assert "rank 3" in _errors(rt, call(M(256, [16, 32]), b, d, d))
+    assert "K mismatch" in _errors(rt, call(a, M(256, [1, 31, 8]), d, d))
+    assert "D is" in _errors(rt, call(a, b, d, M(256, [1, 16, 9])))
+    assert "outside the manifest" in _errors(rt, call(a, b, d, d, num=10**6))
+    assert "negative kernel number" in _errors(rt, call(a, b, d, d, num=-1))
+    assert "split-K" in _errors(rt, call(a, b, d, d, sk=0))
+    assert "not broadcastable" in _errors(rt, call(a, b, M(256, [1, 3, 8]), d, beta=1.0))
+    assert "contiguous" in _errors(rt, call(M(256, [1, 16, 32], [1024, 64, 1]), b, d, d))
+    # aligned kernels reject odd K/N the way can_implement() does
+    odd = call(M(256, [1, 16, 31]), M(256, [1, 31, 8]), d, d)
+    assert "multiples of 8" in _errors(rt, odd)
+
+
+def test_nvte_gemm_argument_checks(rt):
+    M = rt.MemRef
+    a, bt, d = M(256, [1, 16, 32]), M(256, [1, 8, 32]), M(256, [1, 16, 8])
+
+    def call(transa=False, transb=True, alpha=1.0, beta=0.0, C=d, D=d):
+        return lambda lib: lib.nvteGemmF16(*a.args(), transa, *bt.args(), transb, *C.args(), *D.args(),
+                                           0, alpha, beta, 0, 0)
+    assert "transa" in _errors(rt, call(transa=True))
+    assert "transb" in _errors(rt, call(transb=False))
+    assert "alpha must be 1" in _errors(rt, call(alpha=2.0))
+    assert "beta must be 0 or 1" in _errors(rt, call(beta=0.5))
+    assert "C must alias D" in _errors(rt, call(beta=1.0, C=M(512, [1, 16, 8])))
+
+
+def test_other_argument_checks(rt):
+    M = rt.MemRef
+    assert "rank must be 2 or 3" in _errors(rt, lambda lib: lib.nvteLayernormF16(4, M(256, [1, 2, 3, 4]).descriptor, 1e-5))
+    qkv, cu, out = M(256, [2, 64, 2304]), M(256, [3]), M(256, [2, 64, 768])
+    att = lambda q, c, o, heads=12: (lambda lib: lib.nvteBertAttentionF16(*q.args(), *c.args(), *o.args(), 0.125, heads))
+    assert "multiple of 3 * heads" in _errors(rt, att(qkv, cu, out, heads=7))
+    assert "cu_seqlens" in _errors(rt, att(qkv, M(256, [2]), out))
+    assert "Out is" in _errors(rt, att(qkv, cu, M(256, [2, 64, 767])))
+    assert "head size" in _errors(rt, att(M(256, [2, 64, 2304]), cu, out, heads=24))
+    ew = lambda a, b, o: (lambda lib: lib.thrustElementwiseAddF16(*a.args(), *b.args(), *o.args()))
+    assert "only B can broadcast" in _errors(rt, ew(M(256, [3, 1, 3]), M(256, [3, 3, 3]), M(256, [3, 1, 3])))
+    assert "ranks differ" in _errors(rt, ew(M(256, [3, 3]), M(256, [3, 3, 3]), M(256, [3, 3])))
+    ga = lambda i, v, o: (lambda lib: lib.thrustGatherF16(*i.args(), *v.args(), *o.args()))
+    assert "value must be" in _errors(rt, ga(M(256, [2, 4]), M(256, [2, 10, 8]), M(256, [2, 4, 8])))
+    cs = lambda i, o: (lambda lib: lib.thrustCuSeqLenI64(*i.args(), *o.args()))
+    assert "expected 9" in _errors(rt, cs(M(256, [8, 128]), M(256, [8])))
+    assert "fp32 attention" in _errors(rt, lambda lib: lib.nvteBertAttentionF32(*qkv.args(), *cu.args(), *out.args(), 0.125, 12))
+
+
+def test_default_error_mode_aborts(rt):
+    """Reference behaviour: a failed check kills the process (assert / exit(1))."""
+    code = (
+        "import importlib, sys; sys.path.insert(0, %r);"
+        "rt = importlib.import_module('hands-on-mlir_amd.hom_runtime');"
+        "lib = rt.load_runtime();"
+        "m = rt.MemRef(256, [1, 2, 3, 4]);"
+        "lib.nvteLayernormF16(4, m.descriptor, 1e-5); print('survived')" % ROOT)
+    p = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True)
+    assert p.returncode != 0 and "survived" not in p.stdout
+    assert "rank must be 2 or 3" in p.stderr
+
+
+def test_constant_loader_rejects_bad_files(rt, tmp_path, monkeypatch):
+    monkeypatch.setenv("HOM_CONSTANT_DIR", str(tmp_path))
+    (tmp_path / "1.txt").write_text("2 3\n1 2 3 4 5 6\n")
+    (tmp_path / "2.txt").write_text("1 2 3\n1 2 3 4 5\n")
+    assert "cannot open" in _errors(rt, lambda lib: lib.allocConstantNVGPUF16(99))
+    assert "expected 3" in _errors(rt, lambda lib: lib.allocConstantNVGPUF16(1))
+    assert "holds 5 values, expected 6" in _errors(rt, lambda lib: lib.allocConstantNVGPUF16(2))

@@ -1,0 +1,349 @@
+"""Parity of the HIP kernels with the CPU oracle, called through the C-ABI.
+
+Tolerances (written where they are used):
+  GEMM, GEMM+GELU, attention: rtol 1e-3 / atol 1e-2 against the fp32 oracle;
+  layer norm: rtol 2e-3 (atol 1e-3 for outputs near zero);
+  elementwise, gather, cu_seqlens: bit exact.
+"""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+GEMM_TOL = dict(rtol=1e-3, atol=1e-2)
+LN_TOL = dict(rtol=2e-3, atol=1e-3)
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def host(t):
+    torch.cuda.synchronize()
+    return t.cpu().numpy()
+
+
+def assert_close(got, want, rtol, atol, what=""):
+    got = np.asarray(got, np.float64)
+    want = np.asarray(want, np.float64)
+    err = np.abs(got - want)
+    bad = err > atol + rtol * np.abs(want)
+    assert not bad.any(), (f"{what}: {bad.sum()} of {bad.size} outside rtol={rtol} atol={atol}; "
+                           f"max abs err {err.max():.3e} at {np.unravel_index(err.argmax(), err.shape)}")
+
+
+# --------------------------------------------------------------- LayerNorm --
+@pytest.mark.parametrize("shape", [(8, 128, 768), (1024, 768), (3, 5, 1024), (2, 7, 2048), (4, 4096),
+                                   (5, 3, 100), (6, 10), (2, 3, 8200), (1, 1, 8)])
+def test_layernorm_f16_in_place(gpu, rt, oracle, shape):
+    g = np.random.default_rng(sum(shape))
+    x = (g.standard_normal(shape) * 1.5 + 0.3).astype(np.float16)
+    t = dev(x)
+    gpu.nvteLayernormF16(*rt.MemRef.from_tensor(t).args(), 1e-12)
+    assert_close(host(t), oracle.layernorm_f16(x, 1e-12), **LN_TOL, what=f"layernorm {shape}")
+
+
+def test_layernorm_config2_and_large(gpu, rt, oracle, synth):
+    c = synth.add_layernorm()
+    t = dev(c["x"].reshape(8, 128, 768))
+    gpu.nvteLayernormF16(*rt.MemRef.from_tensor(t).args(), c["eps"])
+    assert_close(host(t).reshape(1024, 768), oracle.layernorm_f16(c["x"], c["eps"]), **LN_TOL)
+    # fused residual add + affine (superset), out of place and in place
+    x, r = dev(c["x"]), dev(c["res"])
+    ga, be, out = dev(c["gamma"]), dev(c["beta"]), torch.empty_like(x)
+    M = rt.MemRef.from_tensor
+    gpu.homAddLayernormF16(*M(x).args(), *M(r).args(), *M(ga).args(), *M(be).args(), *M(out).args(), c["eps"])
+    want = oracle.layernorm_f16(c["x"], c["eps"], res=c["res"], gamma=c["gamma"], beta=c["beta"])
+    assert_close(host(out), want, **LN_TOL, what="add+layernorm")
+    gpu.homAddLayernormF16(*M(x).args(), *M(r).args(), *M(ga).args(), *M(be).args(), *M(x).args(), c["eps"])
+    assert np.array_equal(host(x), host(out))
+    # with no residual / affine it is exactly the reference form
+    y = dev(c["x"])
+    gpu.homAddLayernormF16(*M(y).args(), 0, None, 0, None, 0, None, *M(y).args(), c["eps"])
+    assert np.array_equal(host(y).reshape(1024, 768), host(t).reshape(1024, 768))
+    # BERT-large activation size: oracle on the full tensor + invariants
+    g = np.random.default_rng(11)
+    big = (g.standard_normal((32, 512, 1024)) * 2).astype(np.float16)
+    tb = dev(big)
+    gpu.nvteLayernormF16(*M(tb).args(), 1e-12)
+    got = host(tb).astype(np.float64)
+    assert_close(got, oracle.layernorm_f16(big, 1e-12), **LN_TOL)
+    assert np.abs(got.mean(-1)).max() < 2e-3 and np.abs(got.var(-1) - 1).max() < 5e-3
+
+
+def test_layernorm_f32_reference_literal(gpu, rt, oracle, literals):
+    x = np.array(literals["layernorm_2x10"], np.float32).reshape(2, 10)
+    t = dev(x)
+    gpu.nvteLayernormF32(*rt.MemRef.from_tensor(t).args(), 1e-5)
+    assert_close(host(t), oracle.layernorm_f32(x, 1e-5), rtol=1e-5, atol=1e-6)
+    g = np.random.default_rng(5)
+    x = g.standard_normal((2, 33, 768)).astype(np.float32)
+    t = dev(x)
+    gpu.nvteLayernormF32(*rt.MemRef.from_tensor(t).args(), 1e-6)
+    assert_close(host(t), oracle.layernorm_f32(x, 1e-6), rtol=1e-4, atol=1e-5)
+
+
+# ------------------------------------------------------------- elementwise --
+OPS = ["Add", "Sub", "Mul", "Div"]
+
+
+@pytest.mark.parametrize("sfx,dtype", [("F16", np.float16), ("F32", np.float32)])
+def test_elementwise_bit_exact(gpu, rt, oracle, literals, sfx, dtype):
+    g = np.random.default_rng(21)
+    cases = [((3, 3, 3), (3, 1, 3)), ((8, 128, 768), (1, 128, 768)), ((8, 128, 768), (8, 128, 768)),
+             ((4, 6, 40), (1, 1, 40)), ((4, 6, 40), (4, 1, 1)), ((4, 6, 40), (1, 6, 1)),
+             ((5, 7), (5, 7)), ((5, 7), (1, 7)), ((2, 3, 4, 8), (2, 1, 4, 1)), ((1000,), (1000,)),
+             ((3, 5, 17), (1, 1, 1))]
+    for ashape, bshape in cases:
+        a = (g.standard_normal(ashape) + 2.5).astype(dtype)
+        b = (g.standard_normal(bshape) + 2.5).astype(dtype)
+        if ashape == (3, 3, 3) and dtype == np.float32:
+            a = np.array(literals["add_a_3x3x3"], np.float32).reshape(3, 3, 3)
+            b = np.array(literals["add_b_3x1x3"], np.float32).reshape(3, 1, 3)
+        ta, tb = dev(a), dev(b)
+        for op in OPS:
+            out = torch.empty_like(ta)
+            M = rt.MemRef.from_tensor
+            getattr(gpu, f"thrustElementwise{op}{sfx}")(*M(ta).args(), *M(tb).args(), *M(out).args())
+            want = oracle.elementwise(op.lower(), a, b)
+            got = host(out)
+            if op == "Div" and dtype == np.float32:
+                assert_close(got, want, rtol=2e-7, atol=0, what=f"div {ashape}")
+            else:
+                assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), (op, ashape, bshape)
+
+
+def test_gather_and_cu_seqlens_exact(gpu, rt, oracle, literals):
+    g = np.random.default_rng(22)
+    M = rt.MemRef.from_tensor
+    for dtype, sfx, H in [(np.float16, "F16", 768), (np.float32, "F32", 20), (np.float16, "F16", 7)]:
+        table = g.standard_normal((1, 500, H)).astype(dtype)
+        idx = g.integers(0, 500, size=(8, 128)).astype(np.int64)
+        tt, ti = dev(table), dev(idx)
+        out = torch.empty((8, 128, H), dtype=tt.dtype, device="cuda")
+        getattr(gpu, f"thrustGather{sfx}")(*M(ti).args(), *M(tt).args(), *M(out).args())
+        assert np.array_equal(host(out), oracle.gather(idx, table[0]))
+    bs, seq, lens = literals["cuseqlen_bs"], literals["cuseqlen_seq"], literals["cuseqlen_lengths"]
+    mask = np.array([[1 if j < lens[i % 8] else 0 for j in range(seq)] for i in range(bs)], np.int64)
+    for m, fn in [(mask, gpu.thrustCuSeqLenI64), (mask.astype(np.int32), gpu.thrustCuSeqLenI32)]:
+        tm, out = dev(m), torch.full((bs + 1,), -7, dtype=torch.int32, device="cuda")
+        fn(*M(tm).args(), *M(out).args())
+        assert host(out).tolist() == [0, 64, 76, 107, 139, 172, 206, 241, 277, 341, 353, 384, 416,
+                                      449, 483, 518, 554]
+    for bs, seq in [(1, 1), (3, 200), (33, 128), (300, 17)]:
+        m = (g.random((bs, seq)) < 0.6).astype(np.int64)
+        m[0] = 0
+        tm, out = dev(m), torch.empty((bs + 1,), dtype=torch.int32, device="cuda")
+        gpu.thrustCuSeqLenI64(*M(tm).args(), *M(out).args())
+        assert np.array_equal(host(out), oracle.cu_seqlens(m))
+
+
+def test_gelu_kernel(gpu, rt, oracle):
+    x = np.linspace(-9, 9, 4096).astype(np.float16)
+    M = rt.MemRef.from_tensor
+    for form, name in [(0, "erf"), (1, "tanh")]:
+        t, out = dev(x), torch.empty(4096, dtype=torch.float16, device="cuda")
+        gpu.homGeluF16(*M(t).args(), *M(out).args(), form)
+        assert_close(host(out), oracle.gelu(x.astype(np.float64), name), rtol=1e-3, atol=1e-4)
+
+
+# -------------------------------------------------------------------- GEMM --
+def run_gemm(gpu, rt, A, B, C, D_init, num, splitk, alpha=1.0, beta=0.0, act=0, in_place=False):
+    M = rt.MemRef.from_tensor
+    ta, tb = dev(A), dev(B)
+    td = dev(D_init)
+    tc = td if in_place else (dev(C) if C is not None else td)
+    gpu.cutlassGemmF16(*M(ta).args(), False, *M(tb).args(), False, *M(tc).args(), *M(td).args(),
+                       act, alpha, beta, num, splitk)
+    return host(td)
+
+
+def test_gemm_every_manifest_kernel(gpu, rt, oracle):
+    """Every kernel x {tile-aligned, ragged} shapes x {1, 3} K slices."""
+    g = np.random.default_rng(31)
+    shapes8 = [(256, 256, 128), (200, 264, 136), (72, 40, 392)]
+    shapes1 = [(67, 45, 77), (130, 129, 33)]
+    for idx, name, act, align in rt.manifest():
+        epi = "gelu_tanh" if "gelutanh" in name else ("gelu_erf" if act else "linear")
+        for (M_, N_, K_) in (shapes8 if align == 8 else shapes8[:1] + shapes1):
+            A = g.standard_normal((1, M_, K_)).astype(np.float16)
+            B = (g.standard_normal((1, K_, N_)) * 0.1).astype(np.float16)
+            want = oracle.gemm(A[0], B[0], act=epi)
+            for sk in (1, 3):
+                got = run_gemm(gpu, rt, A, B, None, np.zeros((1, M_, N_), np.float16), idx + 1, sk)
+                assert_close(got[0], want, **GEMM_TOL, what=f"{name} {M_}x{N_}x{K_} splitK={sk}")
+
+
+def test_gemm_config1_bias_gelu(gpu, rt, oracle, synth):
+    c = synth.gemm_bias_gelu()
+    for form, act in (("gelu_tanh", 2), ("gelu_erf", 1)):
+        want = oracle.gemm(c["A"][0], c["B"][0], c["bias"][0], beta=1.0, act=form)
+        idx, sk = ctypes.c_int64(), ctypes.c_int32()
+        gpu.homGemmSelect(1024, 3072, 768, act, ctypes.byref(idx), ctypes.byref(sk))
+        got = run_gemm(gpu, rt, c["A"], c["B"], c["bias"], np.zeros((1, 1024, 3072), np.float16),
+                       idx.value + 1, sk.value, beta=1.0)
+        assert_close(got[0], want, **GEMM_TOL, what=f"config 1 {form}")
+        # gemmNum 0: the library picks by the activation argument
+        got0 = run_gemm(gpu, rt, c["A"], c["B"], c["bias"], np.zeros((1, 1024, 3072), np.float16),
+                        0, 1, beta=1.0, act=act)
+        assert_close(got0[0], want, **GEMM_TOL)
+
+
+def test_gemm_residual_in_place_and_batch_folding(gpu, rt, oracle):
+    """out-proj / FFN2 form: beta = 1 with D aliasing C, batch folded into rows."""
+    g = np.random.default_rng(32)
+    b, Mp, K_, N_ = 8, 128, 768, 768
+    A = g.standard_normal((b, Mp, K_)).astype(np.float16)
+    B = (g.standard_normal((1, K_, N_)) * 0.02).astype(np.float16)
+    X = g.standard_normal((b, Mp, N_)).astype(np.float16)
+    want = oracle.gemm(A.reshape(-1, K_), B[0], X.reshape(-1, N_), beta=1.0)
+    for num in (1, 4, 7):
+        for sk in (1, 2, 6):
+            got = run_gemm(gpu, rt, A, B, None, X, num, sk, beta=1.0, in_place=True)
+            assert_close(got.reshape(-1, N_), want, **GEMM_TOL, what=f"in-place kernel {num} splitK {sk}")
+    # [1, M', N] source shared by every batch, alpha/beta other than 1
+    C1 = g.standard_normal((1, Mp, N_)).astype(np.float16)
+    want = oracle.gemm(A.reshape(-1, K_), B[0], C1[0], alpha=0.5, beta=-2.0)
+    got = run_gemm(gpu, rt, A, B, C1, np.zeros((b, Mp, N_), np.float16), 1, 1, alpha=0.5, beta=-2.0)
+    assert_close(got.reshape(-1, N_), want, **GEMM_TOL)
+
+
+def test_gemm_split_k_is_deterministic_and_invariant(gpu, rt, oracle, synth):
+    c = synth.skinny_gemm()  # M=64, K=4096, N=1024
+    want = oracle.gemm(c["A"][0], c["B"][0])
+    outs = {}
+    for sk in (1, 2, 5, 8, 16):
+        a = run_gemm(gpu, rt, c["A"], c["B"], None, np.zeros((1, 64, 1024), np.float16), 4, sk)
+        b = run_gemm(gpu, rt, c["A"], c["B"], None, np.zeros((1, 64, 1024), np.float16), 4, sk)
+        assert np.array_equal(a, b), f"split-K {sk} not reproducible"
+        assert_close(a[0], want, **GEMM_TOL, what=f"skinny splitK={sk}")
+        outs[sk] = a
+    # slices only reassociate the fp32 sum: results agree to fp16 rounding
+    assert np.abs(outs[16].astype(np.float32) - outs[1].astype(np.float32)).max() < 4e-3
+
+
+def test_gemm_exact_cases(gpu, rt, literals):
+    g = np.random.default_rng(33)
+    A = g.standard_normal((1, 128, 128)).astype(np.float16)
+    eye = np.eye(128, dtype=np.float16)[None]
+    for num in (1, 4, 25):
+        assert np.array_equal(run_gemm(gpu, rt, A, eye, None, np.zeros_like(A), num, 1), A)
+        assert np.array_equal(run_gemm(gpu, rt, eye, A, None, np.zeros_like(A), num, 1), A)
+    c = literals["gemm_const"]  # reference driver b.cu: 0.1 x 0.2 over K = 768
+    A = np.full((1, c["m"], c["k"]), c["a"], np.float16)
+    B = np.full((1, c["k"], c["n"]), c["b"], np.float16)
+    out = run_gemm(gpu, rt, A, B, None, np.zeros((1, c["m"], c["n"]), np.float16), 1, 1)
+    assert np.abs(out.astype(np.float64) - c["expect"]).max() < c["tol"]
+
+
+def test_nvte_gemm_path(gpu, rt, oracle):
+    g = np.random.default_rng(34)
+    M = rt.MemRef.from_tensor
+    for (b, Mp, K_, N_, act, beta) in [(8, 128, 768, 2304, 0, 0.0), (8, 128, 768, 3072, 1, 0.0),
+                                       (8, 128, 3072, 768, 0, 1.0), (1, 50, 72, 24, 1, 1.0),
+                                       (2, 9, 37, 21, 0, 0.0)]:
+        A = g.standard_normal((b, Mp, K_)).astype(np.float16)
+        Bt = (g.standard_normal((1, N_, K_)) * 0.05).astype(np.float16)
+        X = g.standard_normal((b, Mp, N_)).astype(np.float16)
+        want = oracle.gemm(A.reshape(-1, K_), Bt[0], X.reshape(-1, N_), beta=beta,
+                           act="gelu_tanh" if act else "linear", b_is_nk=True)
+        ta, tb, td = dev(A), dev(Bt), dev(X)
+        gpu.nvteGemmF16(*M(ta).args(), False, *M(tb).args(), True, *M(td).args(), *M(td).args(),
+                        act, 1.0, beta, 0, 0)
+        assert_close(host(td).reshape(-1, N_), want, **GEMM_TOL, what=f"nvte {Mp}x{N_}x{K_}")
+
+
+def test_ln_gemm_pair(gpu, rt, oracle, literals):
+    """verify.py case: ab = a@b with row stats, then LN(ab) @ c."""
+    a = np.array(literals["verify_a"], np.float16)[None]
+    b = np.array(literals["verify_b"], np.float16)[None]
+    c = np.array(literals["verify_c"], np.float16)[None]
+    M = rt.MemRef.from_tensor
+    ta, tb, tc = dev(a), dev(b), dev(c)
+    ab = torch.zeros((1, 4, 8), dtype=torch.float16, device="cuda")
+    var = torch.zeros((1, 4, 1), dtype=torch.float16, device="cuda")
+    mean = torch.zeros((1, 4, 1), dtype=torch.float16, device="cuda")
+    eps = literals["verify_eps_stats"]
+    gpu.cutlassGemmWithVarMeanF16(*M(ta).args(), *M(tb).args(), *M(ab).args(), *M(ab).args(),
+                                  *M(var).args(), *M(mean).args(), 1.0, 0.0, 0, eps)
+    want_ab = oracle.gemm(a[0], b[0])
+    assert_close(host(ab)[0], want_ab, **GEMM_TOL)
+    v, m = oracle.row_stats(host(ab)[0].astype(np.float32), eps)
+    assert_close(host(var).ravel(), v, rtol=2e-3, atol=1e-3)
+    assert_close(host(mean).ravel(), m, rtol=2e-3, atol=2e-3)
+    out = torch.zeros((1, 4, 16), dtype=torch.float16, device="cuda")
+    gpu.cutlassLayernormGemmF16(*M(ab).args(), *M(tc).args(), *M(out).args(), *M(out).args(),
+                                *M(var).args(), *M(mean).args(), 1.0, 0.0, 0)
+    x = host(ab)[0].astype(np.float64)
+    ln = x * host(var).reshape(4, 1).astype(np.float64) + host(mean).reshape(4, 1).astype(np.float64)
+    assert_close(host(out)[0], ln @ c[0].astype(np.float64), rtol=1e-2, atol=2e-2)
+
+
+# --------------------------------------------------------------- attention --
+def run_attention(gpu, rt, qkv, lens, heads, scale):
+    M = rt.MemRef.from_tensor
+    bs, seq, w = qkv.shape
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    tq, tc = dev(qkv), dev(cu)
+    out = torch.full((bs, seq, w // 3), 7.0, dtype=torch.float16, device="cuda")
+    gpu.nvteBertAttentionF16(*M(tq).args(), *M(tc).args(), *M(out).args(), scale, heads)
+    return host(out), cu
+
+
+def test_attention_config3(gpu, rt, oracle, synth):
+    c = synth.attention()
+    got, cu = run_attention(gpu, rt, c["qkv"], c["lens"], 12, 0.125)
+    want = oracle.attention(c["qkv"], cu, 12, 0.125)
+    assert_close(got, want, **GEMM_TOL, what="attention config 3")
+    for b, n in enumerate(c["lens"]):
+        assert not got[b, n:].any(), "padded query rows must be zeros"
+
+
+@pytest.mark.parametrize("bs,seq,heads,lens", [
+    (2, 64, 2, [64, 1]), (3, 100, 1, [100, 37, 64]), (2, 512, 16, [512, 300]),
+    (4, 128, 12, [0, 128, 65, 33]), (1, 40, 3, [17]), (32, 512, 2, None)])
+def test_attention_shapes_and_edges(gpu, rt, oracle, bs, seq, heads, lens):
+    g = np.random.default_rng(bs * 1000 + seq)
+    qkv = g.standard_normal((bs, seq, 3 * heads * 64)).astype(np.float16)
+    lens = np.array(lens if lens is not None else g.integers(1, seq + 1, size=bs), np.int32)
+    got, cu = run_attention(gpu, rt, qkv, lens, heads, 0.125)
+    assert_close(got, oracle.attention(qkv, cu, heads, 0.125), **GEMM_TOL, what=f"attention {bs}x{seq}x{heads}")
+
+
+def test_attention_layout_onehot(gpu, rt):
+    """Pins the [3][heads][64] interleave: V one-hot in (head 5, d 9)."""
+    heads, seq = 12, 64
+    z = np.zeros((1, seq, 3, heads, 64), np.float16)
+    z[:, :, 2, 5, 9] = 1.0
+    got, _ = run_attention(gpu, rt, z.reshape(1, seq, -1), [seq], heads, 0.125)
+    want = np.zeros((1, seq, heads, 64), np.float16)
+    want[:, :, 5, 9] = 1.0
+    assert np.array_equal(got.reshape(1, seq, heads, 64), want)
+
+
+# ------------------------------------------------------------------ memory --
+def test_alloc_family_and_constant_loader(gpu, rt, tmp_path, monkeypatch):
+    m = gpu.alloc3DMemRefNVGPUF16(2, 3, 4)
+    ptr, sizes, strides = rt.read_descriptor(m)
+    assert m.rank == 3 and sizes == [2, 3, 4] and strides == [12, 4, 1] and ptr != 0
+    gpu.deallocNVGPUF16(m.rank, m.descriptor)
+    m = gpu.alloc1DMemRefNVGPUI32(9)
+    assert rt.read_descriptor(m)[1:] == ([9], [1])
+    gpu.deallocNVGPUI32(m.rank, m.descriptor)
+    vals = np.arange(24, dtype=np.float32) * 0.37 - 3
+    (tmp_path / "5.txt").write_text("2 3 4\n" + " ".join(repr(float(v)) for v in vals) + "\n")
+    monkeypatch.setenv("HOM_CONSTANT_DIR", str(tmp_path))
+    for fn, dt in [(gpu.allocConstantNVGPUF16, torch.float16), (gpu.allocConstantNVGPUF32, torch.float32)]:
+        m = fn(5)
+        ptr, sizes, _ = rt.read_descriptor(m)
+        assert sizes == [2, 3, 4]
+        out = torch.empty(24, dtype=dt, device="cuda")
+        hip = ctypes.CDLL("libamdhip64.so")
+        hip.hipMemcpy.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int]
+        assert hip.hipMemcpy(out.data_ptr(), ptr, 24 * out.element_size(), 3) == 0
+        want = vals.astype(np.float16 if dt == torch.float16 else np.float32)
+        assert np.array_equal(host(out), want)
+        gpu.deallocNVGPUF16(m.rank, m.descriptor)
