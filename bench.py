@@ -1,0 +1,181 @@
+#!/usr/bin/env python3
+"""Headline benchmark: BERT-base fp16 encoder, batch 8 x seq 128, sequences/s.
+
+A "step" is one forward of the 12-layer encoder (embedding gather + add + layer
+norm, then per layer QKV GEMM, attention, out-proj GEMM + residual, layer norm,
+FFN1 GEMM + GELU, FFN2 GEMM + residual, layer norm) over one resident synthetic
+batch, driven by the C++ host driver through the C-ABI and replayed as a HIP
+graph.  Inputs and weights are in HBM before the timed region starts.
+
+Prints one JSON line.  Besides the contract fields it carries
+  roofline      FFN1 GEMM + bias + GELU (M=1024, K=768, N=3072), timed with HIP
+                events on the stream it is launched on;
+  cpu_baseline  the single-threaded fp32 restatement of the reference's CPU
+                lowering, timed on a bounded sample of the same workload;
+  kernels       achieved rates of the other kernels on the path (informative).
+"""
+import argparse
+import ctypes
+import importlib
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "oracle")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+METRIC = "BERT-base fp16 seqs/sec @b8 s128; GEMM+GELU TFLOPS and % of MFMA peak"
+PEAK_FP16_TFLOPS = 2500.0   # MI355X dense fp16 MFMA
+PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
+
+
+def cpu_baseline(synth, seconds_hint=20.0):
+    """One encoder layer of the CPU lowering (fp32, one thread) on b2 x s128."""
+    import numpy as np
+    import oracle  # test/benchmark infrastructure: the CPU port
+    base = oracle.baseline()
+    P = lambda a: a.ctypes.data_as(ctypes.c_void_p)
+    bs, seq, H, heads, F = 4, 128, 768, 12, 3072
+    g = np.random.default_rng(0)
+    rows = bs * seq
+    x = g.standard_normal((rows, H)).astype(np.float32)
+    w = {k: (g.standard_normal(s) * 0.02).astype(np.float32)
+         for k, s in (("qkv", (H, 3 * H)), ("o", (H, H)), ("1", (H, F)), ("2", (F, H)))}
+    qkv = np.empty((rows, 3 * H), np.float32)
+    attn = np.empty((rows, H), np.float32)
+    scores = np.empty((seq, seq), np.float32)
+    f = np.empty((rows, F), np.float32)
+    t0, t1 = np.empty_like(f), np.empty_like(f)
+    gel = np.empty_like(f)
+    h1 = np.empty((rows, H), np.float32)
+    tmp = np.empty((rows, H), np.float32)
+    lens = np.array([128, 80, 100, 60], np.int32)
+    start = time.perf_counter()
+    base.hom_cpu_matmul_add_f32(P(x), P(w["qkv"]), None, P(qkv), 1, rows, 3 * H, H, 1, 1)
+    base.hom_cpu_attention_f32(P(qkv), P(lens), P(attn), P(scores), bs, seq, heads, H // heads, 0.125)
+    base.hom_cpu_matmul_add_f32(P(attn), P(w["o"]), P(x), P(h1), 1, rows, H, H, 1, 0)
+    base.hom_cpu_layernorm_tosa_f32(P(h1), P(tmp), rows, H, 1e-12)
+    base.hom_cpu_matmul_add_f32(P(h1), P(w["1"]), None, P(f), 1, rows, F, H, 1, 1)
+    base.hom_cpu_gelu_tosa_f32(P(f), P(gel), P(t0), P(t1), rows * F)
+    base.hom_cpu_matmul_add_f32(P(gel), P(w["2"]), P(h1), P(x), 1, rows, H, F, 1, 0)
+    base.hom_cpu_layernorm_tosa_f32(P(x), P(tmp), rows, H, 1e-12)
+    layer_s = time.perf_counter() - start
+    return {"value": bs / (layer_s * 12), "unit": "sequences/s", "cores": 1, "kind": "port",
+            "host_cores": os.cpu_count(),
+            "sample": f"1 of 12 encoder layers on 4 of 8 sequences (b4 s128) in {layer_s:.1f} s, "
+                      "scaled x12 layers; fp32, one thread, loop order of matmulAddF32"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--eager", action="store_true", help="launch every call instead of replaying a HIP graph")
+    ap.add_argument("--gemm-mode", type=int, default=1,
+                    help="0 nvteGemmF16 path, 1 cutlassGemmF16 + tuned table, 2 + live autotune")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this path runs on one GPU; --gpus N with N > 1 is not supported "
+                 "(the workload shards by batch with no exchange step, see DESIGN.md)")
+
+    import numpy as np
+    import torch
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    rt = importlib.import_module("hands-on-mlir_amd.hom_runtime")
+    synth = importlib.import_module("hands-on-mlir_amd.synth")
+    bert = importlib.import_module("hands-on-mlir_amd.bert")
+    drv = rt.load_driver()  # fails loudly when the HIP libraries are missing
+    lib = rt.load_runtime()
+
+    model = synth.bert_encoder()
+    d = model["dims"]
+    enc = bert.BertEncoder(d["layers"], d["hidden"], d["heads"], d["ffn"], d["bs"], d["seq"], d["vocab"],
+                           gemm_mode=args.gemm_mode, gelu_form="erf")
+    enc.load(model)
+    enc.set_inputs(ids=model["ids"], mask=model["mask"])
+    torch.cuda.synchronize()
+    t_wall = time.perf_counter()
+    ms = enc.time(args.steps, args.warmup, graph=not args.eager)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t_wall
+    choices = enc.gemm_choices()
+    names = {i + 1: n for i, n, _, _ in rt.manifest()}
+    enc.close()
+    seqs_per_s = d["bs"] / (ms * 1e-3)
+    flops_forward = 12 * (2 * 1024 * 7077888 + 402653184)
+
+    # dominant kernel: FFN1 GEMM + bias + GELU, BERT-base shape
+    M, K, N = 1024, 768, 3072
+    idx, sk = ctypes.c_int64(), ctypes.c_int32()
+    lib.homGemmSelect(M, N, K, 2, ctypes.byref(idx), ctypes.byref(sk))
+    g_ms = drv.homTimeGemm(M, N, K, 2, 1, idx.value + 1, sk.value, 2000, 50)
+    g_flops = 2.0 * M * N * K
+    achieved = g_flops / (g_ms * 1e-3) / 1e12
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "traffic.json")
+    if os.path.exists(tpath):
+        traffic = json.load(open(tpath)).get("gemm_bias_gelu_1024x3072x768")
+
+    def gbs(nbytes, t_ms):
+        return nbytes / (t_ms * 1e-3) / 1e9
+
+    kernels = {}
+    ln_ms = drv.homTimeLayernorm(1024, 768, 0, 2000, 50)
+    kernels["layernorm_1024x768_inplace"] = {"us": ln_ms * 1e3, "GB/s": gbs(2 * 1024 * 768 * 2, ln_ms)}
+    aln_ms = drv.homTimeLayernorm(1024, 768, 1, 2000, 50)
+    kernels["add_layernorm_1024x768"] = {"us": aln_ms * 1e3, "GB/s": gbs(4721664, aln_ms)}
+    ln5_ms = drv.homTimeLayernorm(16384, 1024, 0, 500, 20)
+    kernels["layernorm_16384x1024_inplace"] = {"us": ln5_ms * 1e3, "GB/s": gbs(2 * 16384 * 1024 * 2, ln5_ms),
+                                               "frac_hbm": gbs(2 * 16384 * 1024 * 2, ln5_ms) / PEAK_HBM_GBS}
+    add5_ms = drv.homTimeElementwiseAdd(16384, 1024, 500, 20)
+    kernels["add_16384x1024"] = {"us": add5_ms * 1e3, "GB/s": gbs(3 * 16384 * 1024 * 2, add5_ms),
+                                 "frac_hbm": gbs(3 * 16384 * 1024 * 2, add5_ms) / PEAK_HBM_GBS}
+    lens = (ctypes.c_int32 * 8)(*[int(x) for x in synth.attention()["lens"]])
+    at_ms = drv.homTimeAttention(8, 128, 12, lens, 2000, 50)
+    kernels["attention_b8_s128_h12"] = {"us": at_ms * 1e3, "GB/s": gbs(6291492, at_ms),
+                                        "dense_TFLOP/s": 402653184 / (at_ms * 1e-3) / 1e12}
+    for (m, n, k, act, tag) in [(16384, 4096, 1024, 1, "gemm_gelu_16384x4096x1024"),
+                                (16384, 1024, 4096, 0, "gemm_16384x1024x4096"),
+                                (64, 1024, 4096, 0, "gemm_skinny_64x1024x4096")]:
+        lib.homGemmSelect(m, n, k, act, ctypes.byref(idx), ctypes.byref(sk))
+        t = drv.homTimeGemm(m, n, k, act, 0, idx.value + 1, sk.value, 100 if m > 1024 else 1000, 10)
+        tf = 2.0 * m * n * k / (t * 1e-3) / 1e12
+        kernels[tag] = {"us": t * 1e3, "TFLOP/s": tf, "frac_mfma": tf / PEAK_FP16_TFLOPS,
+                        "kernel": names[idx.value + 1], "splitK": sk.value}
+
+    out = {
+        "metric": METRIC, "value": seqs_per_s, "unit": "sequences/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "BERT-base encoder fp16, 12 layers, hidden 768, 12 heads, FFN 3072, "
+                               "batch 8 x seq 128, padding mask (configs[3])",
+                   "launch": "eager C-ABI calls" if args.eager else "HIP graph replay of the C-ABI call list",
+                   "gemm_mode": args.gemm_mode,
+                   "gemm_kernels": {k: {"kernel": names.get(v[0], "library-selected"), "splitK": v[1]}
+                                    for k, v in choices.items()}},
+        "encoder_TFLOP/s": flops_forward / (ms * 1e-3) / 1e12,
+        "wall_s_timed_region": wall,
+        "roofline": {"kernel": names[idx.value + 1] if False else None, "bound": "mfma",
+                     "achieved": achieved, "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": achieved / PEAK_FP16_TFLOPS, "traffic": traffic,
+                     "us_per_launch": g_ms * 1e3, "flops_per_launch": g_flops,
+                     "shape": "M=1024 K=768 N=3072 bias + tanh-GELU"},
+        "kernels": kernels,
+    }
+    lib.homGemmSelect(M, N, K, 2, ctypes.byref(idx), ctypes.byref(sk))
+    out["roofline"]["kernel"] = names[idx.value + 1]
+    out["roofline"]["splitK"] = sk.value
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(synth)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -485,6 +485,31 @@ DRV_EXPORT double homTimeGemm(int64_t M, int64_t N, int64_t K, int64_t act,
   return ms;
 }
 
+// Same through nvteGemmF16 (B given as [1, N, K]); the library picks the kernel.
+DRV_EXPORT double homTimeGemmNvte(int64_t M, int64_t N, int64_t K, int64_t act,
+                                  int iters, int warmup) {
+  Tensor a, b, d;
+  a.m = alloc3DMemRefNVGPUF16(1, int32_t(M), int32_t(K));
+  b.m = alloc3DMemRefNVGPUF16(1, int32_t(N), int32_t(K));
+  d.m = alloc3DMemRefNVGPUF16(1, int32_t(M), int32_t(N));
+  fillRandomF16(a.data(), M * K, 1.0f, 1);
+  fillRandomF16(b.data(), K * N, 0.02f, 2);
+  double ms;
+  {
+    Timer t;
+    ms = t.run(
+        [&] {
+          nvteGemmF16(3, a.m.descriptor, false, 3, b.m.descriptor, true, 3,
+                      d.m.descriptor, 3, d.m.descriptor, act, 1.0f, 0.0f, 0, 0);
+        },
+        iters, warmup);
+  }
+  a.release();
+  b.release();
+  d.release();
+  return ms;
+}
+
 // In-place layer norm (reference form) when fused == 0; residual add + affine
 // layer norm (homAddLayernormF16) when fused != 0.
 DRV_EXPORT double homTimeLayernorm(int64_t rows, int64_t hidden, int fused,

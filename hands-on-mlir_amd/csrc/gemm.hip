@@ -8,28 +8,39 @@
 // (python/gemm_generator.py:237-278, python/hom_manifest.py:503-533) and the
 // cuBLASLt call behind nvteGemmF16 (include/NVGPUKernels/GemmRunner.h:404-425).
 //
-// Kernel structure
+// Common structure
 //  * one workgroup of WM x WN wavefronts computes a BM x BN tile of D; every
 //    wavefront owns a (BM/WM) x (BN/WN) sub-tile made of 32x32 MFMA blocks
 //    (v_mfma_f32_32x32x16_f16: 64 lanes x 8 halves per operand, 16 fp32
 //    accumulators per lane);
-//  * K is walked in BK slabs that are staged global -> registers -> LDS with
-//    two LDS buffers, so the loads of slab k+1 overlap the MFMAs of slab k;
-//  * A is kept K-contiguous in LDS (row padded by 16 bytes, which makes the
-//    128-bit fragment reads bank-conflict free).  Row-major B has N
-//    contiguous, but an MFMA operand wants 8 consecutive k per lane: while
-//    staging, each thread interleaves two consecutive k rows into (k, k+1)
-//    half2 pairs, and a fragment is then four conflict-free 32-bit reads;
 //  * the MFMA is issued with the operands swapped (B fragment first), i.e. it
 //    produces the transposed block, so each lane ends up with 4 consecutive
 //    columns of one row of D and the epilogue can use 64-bit accesses;
-//  * split-K: gridDim.y slices of K.  Each slice stores its fp32 partial tile
-//    to a workspace and bumps a per-tile arrival counter; whichever slice
-//    arrives last sums all partials in slice order (deterministic) and runs the
-//    epilogue, then clears the counter for the next launch.  Nothing spins.
+//  * split-K: gridDim.y slices of K each store their fp32 partial tile to a
+//    workspace; a second, small kernel sums the slices in slice order
+//    (deterministic, fp32) and runs the epilogue.  Nothing spins or fences;
 //  * workgroup ids are remapped so that each of the 8 XCDs (which receive
 //    consecutive ids round-robin and have private L2s) works on a contiguous
 //    run of tiles.
+//
+// Two main-loop families
+//  * "dma" kernels (the fast path, aligned problems): K is walked in 64-wide
+//    slabs through an NS-deep ring of LDS buffers filled by
+//    buffer_load_dwordx4 ... lds, i.e. global memory -> LDS without passing
+//    through registers.  The loads of slab k+NS-1 are in flight while slab k is
+//    multiplied, which is what hides HBM/L2 latency when only one or two
+//    workgroups fit a CU.  Out-of-range rows/columns/k are given an offset
+//    beyond the buffer descriptor's size, for which the hardware writes zeros.
+//    LDS rows are not padded (the DMA writes 1 KiB contiguous per wavefront);
+//    bank conflicts are avoided by permuting 16-byte chunks inside a row, which
+//    costs nothing because every lane chooses its own global address.
+//    A (and B when it is [N, K]) fragments are 128-bit LDS reads.  Row-major B
+//    has N contiguous while an MFMA operand wants 8 consecutive k per lane:
+//    those fragments are read with ds_read_b64_tr_b16, which transposes 4 k-rows
+//    x 16 columns across a group of 16 lanes.
+//  * "staged" kernels (any shape / alignment, and the first bring-up path):
+//    global -> registers -> LDS with two LDS buffers and 32-wide slabs; row-major
+//    B is interleaved into (k, k+1) half2 pairs while it is staged.
 #include "kernels.h"
 
 namespace hom {
@@ -37,21 +48,22 @@ namespace {
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef _Float16 half4 __attribute__((ext_vector_type(4)));
-typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 typedef float float16v __attribute__((ext_vector_type(16)));
 typedef float float4v __attribute__((ext_vector_type(4)));
 typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
+typedef short short4v __attribute__((ext_vector_type(4)));
 
 constexpr int kWave = 64;
 constexpr int kNumXcd = 8;
+
+#define HOM_LDS_PTR(p) ((__attribute__((address_space(3))) void *)(p))
 
 struct GemmParams {
   const _Float16 *A;
   const _Float16 *B;
   const _Float16 *C;
   _Float16 *D;
-  float *workspace;    // split-K partial tiles
-  uint32_t *counters;  // split-K arrival counters, one per output tile
+  float *workspace; // split-K partial tiles (null when gridDim.y == 1)
   int M, N, K;
   int64_t lda, ldb, ldc, ldd;
   int cRowPeriod;
@@ -77,38 +89,430 @@ template <int EPI> __device__ __forceinline__ float activate(float v) {
   return v;
 }
 
+// XCD-contiguous tile id for this workgroup.
+__device__ __forceinline__ int tileForBlock(int nTiles) {
+  const int pid = blockIdx.x;
+  const int q = nTiles / kNumXcd, r = nTiles % kNumXcd;
+  const int xcd = pid % kNumXcd, loc = pid / kNumXcd;
+  return xcd * q + (xcd < r ? xcd : r) + loc;
+}
+
+// Tile id -> (tile row, tile column).  Ids walk groups of kGroupM tile rows
+// column by column, so that the workgroups running at the same time on one XCD
+// cover a compact block of D and share both A rows and B columns in that XCD's
+// L2 instead of streaming all of B for every tile row.
+constexpr int kGroupM = 8;
+__device__ __forceinline__ void tileCoords(int tile, int tilesM, int tilesN,
+                                           int *tileM, int *tileN) {
+  const int groupSize = kGroupM * tilesN;
+  const int g = tile / groupSize;
+  const int firstM = g * kGroupM;
+  const int rows = tilesM - firstM < kGroupM ? tilesM - firstM : kGroupM;
+  const int inGroup = tile - g * groupSize;
+  *tileM = firstM + inGroup % rows;
+  *tileN = inGroup / rows;
+}
+
+// Accumulator layout shared by every kernel here (transposed 32x32 block):
+// accumulator e of lane l is column 8*(e/4) + 4*(l/32) + e%4, row l%32.
+template <int MI, int NI, int WTM, int WTN, int EPI, int VEC>
+__device__ __forceinline__ void epilogueStore(const GemmParams &p,
+                                              float16v (&acc)[MI][NI], int m0,
+                                              int n0, int waveM, int waveN,
+                                              int lane) {
+  const int l32 = lane % 32, kb = lane / 32;
+  const bool useC = p.beta != 0.f;
+#pragma unroll
+  for (int i = 0; i < MI; i++) {
+    const int m = m0 + waveM * WTM + i * 32 + l32;
+    if (m >= p.M)
+      continue;
+    const int64_t cRow = int64_t(m % p.cRowPeriod) * p.ldc;
+    const int64_t dRow = int64_t(m) * p.ldd;
+#pragma unroll
+    for (int j = 0; j < NI; j++) {
+#pragma unroll
+      for (int g = 0; g < 4; g++) {
+        const int n = n0 + waveN * WTN + j * 32 + g * 8 + kb * 4;
+        if (VEC == 8) {
+          if (n >= p.N)
+            continue;
+          float c[4] = {0.f, 0.f, 0.f, 0.f};
+          if (useC) {
+            const half4 cv = *reinterpret_cast<const half4 *>(p.C + cRow + n);
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+              c[e] = float(cv[e]);
+          }
+          half4 o;
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            float v = p.alpha * acc[i][j][g * 4 + e];
+            if (useC)
+              v += p.beta * c[e];
+            o[e] = _Float16(activate<EPI>(v));
+          }
+          *reinterpret_cast<half4 *>(p.D + dRow + n) = o;
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            if (n + e < p.N) {
+              float v = p.alpha * acc[i][j][g * 4 + e];
+              if (useC)
+                v += p.beta * float(p.C[cRow + n + e]);
+              p.D[dRow + n + e] = _Float16(activate<EPI>(v));
+            }
+          }
+        }
+      }
+    }
+  }
+}
+
+// Partial tile of one K slice -> workspace, in accumulator order (coalesced
+// 128-bit stores; the reduce kernel uses the same thread -> element mapping).
+template <int MI, int NI, int THREADS>
+__device__ __forceinline__ void storePartial(const GemmParams &p,
+                                             float16v (&acc)[MI][NI], int tile,
+                                             int slice, int numSlices,
+                                             int tid) {
+  constexpr int ACC_V4 = MI * NI * 4;
+  float4v *mine = reinterpret_cast<float4v *>(p.workspace) +
+                  (int64_t(tile) * numSlices + slice) * (ACC_V4 * THREADS);
+#pragma unroll
+  for (int i = 0; i < MI; i++)
+#pragma unroll
+    for (int j = 0; j < NI; j++)
+#pragma unroll
+      for (int g = 0; g < 4; g++) {
+        float4v v;
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+          v[e] = acc[i][j][g * 4 + e];
+        mine[((i * NI + j) * 4 + g) * THREADS + tid] = v;
+      }
+}
+
+template <int BM, int BN, int WM, int WN, int EPI, int VEC>
+__global__ __launch_bounds__(WM *WN *kWave) void splitKReduceKernel(
+    GemmParams p, int numSlices) {
+  constexpr int THREADS = WM * WN * kWave;
+  constexpr int WTM = BM / WM, WTN = BN / WN;
+  constexpr int MI = WTM / 32, NI = WTN / 32;
+  constexpr int ACC_V4 = MI * NI * 4;
+  const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+  const int tile = blockIdx.x;
+  int tileM, tileN;
+  tileCoords(tile, p.tilesM, p.tilesN, &tileM, &tileN);
+  float16v acc[MI][NI];
+#pragma unroll
+  for (int i = 0; i < MI; i++)
+#pragma unroll
+    for (int j = 0; j < NI; j++)
+#pragma unroll
+      for (int e = 0; e < 16; e++)
+        acc[i][j][e] = 0.f;
+  const float4v *ws = reinterpret_cast<const float4v *>(p.workspace) +
+                      int64_t(tile) * numSlices * (ACC_V4 * THREADS);
+  for (int s = 0; s < numSlices; s++) {
+    const float4v *part = ws + int64_t(s) * (ACC_V4 * THREADS);
+#pragma unroll
+    for (int i = 0; i < MI; i++)
+#pragma unroll
+      for (int j = 0; j < NI; j++)
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+          const float4v v = part[((i * NI + j) * 4 + g) * THREADS + tid];
+#pragma unroll
+          for (int e = 0; e < 4; e++)
+            acc[i][j][g * 4 + e] += v[e];
+        }
+  }
+  epilogueStore<MI, NI, WTM, WTN, EPI, VEC>(p, acc, tileM * BM, tileN * BN,
+                                            wave / WN, wave % WN, lane);
+}
+
+// ===================================================================== dma ==
+// Swizzles (in units of 16-byte chunks / 64-byte groups inside an LDS row).
+// K-contiguous tiles (A, and B given as [N, K]): rows of 128 bytes = 8 chunks;
+// chunk c of row r lives at position c ^ ((r >> 1) & 7), which makes the
+// 128-bit fragment reads of 16 consecutive rows hit 16 distinct bank groups.
+__device__ __forceinline__ int swzK(int row, int chunk) {
+  return chunk ^ ((row >> 1) & 7);
+}
+// Row-major B tiles: a transposing read touches rows k..k+3 and k+8..k+11, 64
+// bytes of each; 64-byte group g of row k lives at position g ^ f(k).
+template <int BN> __device__ __forceinline__ int swzN(int k, int group) {
+  if (BN == 64)
+    return group ^ ((k >> 1) & 1);
+  return group ^ (k & 3);
+}
+
+template <int BM, int BN, int WM, int WN, int NS, int EPI, bool B_NK>
+__global__ __launch_bounds__(WM *WN *kWave) void gemmDmaKernel(GemmParams p) {
+  // The body uses buffer-descriptor builtins whose types exist only for the
+  // GPU target; the host pass needs just the (empty) stub to launch through.
+#if defined(__HIP_DEVICE_COMPILE__)
+  constexpr int BK = 64;
+  constexpr int THREADS = WM * WN * kWave;
+  constexpr int NW = WM * WN;
+  constexpr int WTM = BM / WM, WTN = BN / WN;
+  constexpr int MI = WTM / 32, NI = WTN / 32;
+  constexpr int A_BYTES = BM * BK * 2, B_BYTES = BN * BK * 2;
+  constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
+  constexpr int A_INSTR = A_BYTES / 1024, B_INSTR = B_BYTES / 1024;
+  static_assert(A_INSTR % NW == 0 && B_INSTR % NW == 0,
+                "tile must split evenly over the wavefronts");
+  constexpr int A_PER_W = A_INSTR / NW, B_PER_W = B_INSTR / NW;
+  constexpr int LOADS_PER_TILE = A_PER_W + B_PER_W; // per wavefront
+  constexpr int B_ROW_BYTES = B_NK ? 128 : BN * 2;
+  constexpr int B_ROWS_PER_INSTR = 1024 / B_ROW_BYTES;
+  static_assert((NS - 2) * LOADS_PER_TILE < 64, "vmcnt is a 6-bit counter");
+
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+
+  const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+  const int waveM = wave / WN, waveN = wave % WN;
+  const int l32 = lane % 32, kb = lane / 32;
+
+  const int nTiles = p.tilesM * p.tilesN;
+  const int tile = tileForBlock(nTiles);
+  int tileM, tileN;
+  tileCoords(tile, p.tilesM, p.tilesN, &tileM, &tileN);
+  const int m0 = tileM * BM, n0 = tileN * BN;
+  const int slice = blockIdx.y, numSlices = gridDim.y;
+  const int kTiles = (p.K + BK - 1) / BK;
+  const int ktBegin = slice * p.kTilesPerSlice;
+  int ktEnd = ktBegin + p.kTilesPerSlice;
+  if (ktEnd > kTiles)
+    ktEnd = kTiles;
+
+  // Buffer descriptors based at this tile's first row (A) / first row or
+  // column block (B), so 32-bit offsets suffice for any matrix size.  Offsets
+  // at or beyond num_records read as zero.
+  constexpr uint32_t kOob = 0x80000000u;
+  auto clampBytes = [](int64_t b) -> int32_t {
+    return b > 0x7fffffffLL ? 0x7fffffff : (b < 0 ? 0 : int32_t(b));
+  };
+  const _Float16 *aBase = p.A + int64_t(m0) * p.lda;
+  const int64_t aBytes = (int64_t(p.M - m0) * p.lda) * 2;
+  const auto rsrcA = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<_Float16 *>(aBase), 0, clampBytes(aBytes), 0x00020000);
+  const _Float16 *bBase = B_NK ? p.B + int64_t(n0) * p.ldb : p.B;
+  const int64_t bBytes =
+      B_NK ? (int64_t(p.N - n0) * p.ldb) * 2 : (int64_t(p.K) * p.ldb) * 2;
+  const auto rsrcB = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<_Float16 *>(bBase), 0, clampBytes(bBytes), 0x00020000);
+  // Row-major B deeper than 2 GiB would overflow the 32-bit offset; the host
+  // rejects such problems for these kernels.
+
+  // ---- per-lane source offsets (bytes), constant over the K walk ----
+  uint32_t aOff[A_PER_W];
+  int aCol[A_PER_W];
+#pragma unroll
+  for (int i = 0; i < A_PER_W; i++) {
+    const int instr = wave * A_PER_W + i;
+    const int r = instr * 8 + lane / 8;
+    const int c = swzK(r, lane % 8); // logical chunk stored at this position
+    aCol[i] = c * 8;
+    aOff[i] = (m0 + r < p.M) ? uint32_t((int64_t(r) * p.lda + c * 8) * 2) : kOob;
+  }
+  uint32_t bOff[B_PER_W];
+  int bK[B_PER_W]; // NK: column offset in k; KN: row (k) inside the slab
+#pragma unroll
+  for (int i = 0; i < B_PER_W; i++) {
+    const int instr = wave * B_PER_W + i;
+    if (B_NK) {
+      const int r = instr * 8 + lane / 8;
+      const int c = swzK(r, lane % 8);
+      bK[i] = c * 8;
+      bOff[i] = (n0 + r < p.N) ? uint32_t((int64_t(r) * p.ldb + c * 8) * 2) : kOob;
+    } else {
+      constexpr int CHUNKS = B_ROW_BYTES / 16;
+      const int k = instr * B_ROWS_PER_INSTR + lane / CHUNKS;
+      const int pc = lane % CHUNKS; // physical chunk
+      const int g = swzN<BN>(k, pc / 4);
+      const int n = (g * 4 + pc % 4) * 8;
+      bK[i] = k;
+      bOff[i] = (n0 + n < p.N) ? uint32_t((int64_t(k) * p.ldb + n0 + n) * 2) : kOob;
+    }
+  }
+
+  auto issue = [&](int kt, int stage) {
+    unsigned char *sA = smem + stage * STAGE_BYTES;
+    unsigned char *sB = sA + A_BYTES;
+    const int k0 = kt * BK;
+    const bool live = kt < ktEnd;
+#pragma unroll
+    for (int i = 0; i < A_PER_W; i++) {
+      const uint32_t off = (live && k0 + aCol[i] < p.K && aOff[i] != kOob)
+                               ? aOff[i] + uint32_t(k0) * 2u
+                               : kOob;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(
+          rsrcA, HOM_LDS_PTR(sA + (wave * A_PER_W + i) * 1024), 16, off, 0, 0, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < B_PER_W; i++) {
+      uint32_t off;
+      if (B_NK)
+        off = (live && k0 + bK[i] < p.K && bOff[i] != kOob)
+                  ? bOff[i] + uint32_t(k0) * 2u
+                  : kOob;
+      else
+        off = (live && k0 + bK[i] < p.K && bOff[i] != kOob)
+                  ? bOff[i] + uint32_t(int64_t(k0) * p.ldb * 2)
+                  : kOob;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(
+          rsrcB, HOM_LDS_PTR(sB + (wave * B_PER_W + i) * 1024), 16, off, 0, 0, 0);
+    }
+  };
+
+  float16v acc[MI][NI];
+#pragma unroll
+  for (int i = 0; i < MI; i++)
+#pragma unroll
+    for (int j = 0; j < NI; j++)
+#pragma unroll
+      for (int e = 0; e < 16; e++)
+        acc[i][j][e] = 0.f;
+
+  // ---- fragment addresses (bytes inside a stage), constant over the walk ----
+  // A: row r = waveM*WTM + i*32 + l32, logical chunk kk*2 + kb.
+  const int aRow0 = waveM * WTM + l32;
+  // B (row-major): transposing read.  Source lane L = lane%16 of a 16-lane
+  // group supplies row kbase + L/4, 4 columns at (L%4)*4; the group's 16 columns
+  // start at ((lane%32)/16)*16 of the 32-wide block.
+  const int trRow = (lane % 16) / 4;
+  const int trCol = ((lane % 32) / 16) * 16 + (lane % 4) * 4;
+
+  // Fragments of one 16-wide k step of a stage, into registers.
+  auto loadFrags = [&](int stage, int kk, half8 (&fa)[MI], half8 (&fb)[NI]) {
+    const unsigned char *sA = smem + stage * STAGE_BYTES;
+    const unsigned char *sB = sA + A_BYTES;
+#pragma unroll
+    for (int i = 0; i < MI; i++) {
+      const int r = aRow0 + i * 32;
+      fa[i] = *reinterpret_cast<const half8 *>(sA + r * 128 +
+                                               swzK(r, kk * 2 + kb) * 16);
+    }
+    if (B_NK) {
+#pragma unroll
+      for (int j = 0; j < NI; j++) {
+        const int r = waveN * WTN + j * 32 + l32;
+        fb[j] = *reinterpret_cast<const half8 *>(sB + r * 128 +
+                                                 swzK(r, kk * 2 + kb) * 16);
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < NI; j++) {
+        const int n = waveN * WTN + j * 32 + trCol;
+        short4v t[2];
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+          const int k = kk * 16 + kb * 8 + h * 4 + trRow;
+          const unsigned char *src =
+              sB + k * B_ROW_BYTES + swzN<BN>(k, n / 32) * 64 + (n % 32) * 2;
+          t[h] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+              (__attribute__((address_space(3))) short4v *)(src));
+        }
+        typedef short short8v __attribute__((ext_vector_type(8)));
+        short8v both;
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          both[e] = t[0][e];
+          both[4 + e] = t[1][e];
+        }
+        fb[j] = __builtin_bit_cast(half8, both);
+      }
+    }
+  };
+  auto mfmaStep = [&](half8 (&fa)[MI], half8 (&fb)[NI]) {
+#pragma unroll
+    for (int i = 0; i < MI; i++)
+#pragma unroll
+      for (int j = 0; j < NI; j++)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[j], fa[i],
+                                                           acc[i][j], 0, 0, 0);
+  };
+
+  // ---- main loop: NS-deep ring of slabs, one barrier per slab ----
+  // Every wavefront issues exactly LOADS_PER_TILE DMA loads per slab (slabs past
+  // the end are all out of range and write zeros), so "slab i+1 has landed" is
+  // vmcnt <= (NS-2) * LOADS_PER_TILE once slabs up to i+NS-1 have been issued.
+  // Inside a slab the fragments of k step kk+1 are fetched from LDS before the
+  // MFMAs of step kk are issued (two register sets), and the barrier that frees
+  // the slab's LDS buffer sits between the last fragment fetch and the last
+  // MFMA group, so the matrix core keeps running while the wavefronts
+  // synchronise, refill the ring and fetch the next slab's first fragments.
+  // The waits and the barrier are one opaque asm statement with a memory
+  // clobber: the compiler may not move LDS reads or DMA issues across it.
+  constexpr int kInFlight = (NS - 2) * LOADS_PER_TILE;
+  constexpr int KSTEPS = BK / 16;
+  half8 fa[2][MI], fb[2][NI];
+#pragma unroll
+  for (int s = 0; s < NS - 1; s++)
+    issue(ktBegin + s, s);
+  const int nk = ktEnd - ktBegin;
+  if (nk > 0) {
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(kInFlight) : "memory");
+    issue(ktBegin + NS - 1, NS - 1);
+    loadFrags(0, 0, fa[0], fb[0]);
+    for (int i = 0; i < nk; i++) {
+      const int cur = i % NS;
+#pragma unroll
+      for (int kk = 0; kk < KSTEPS - 1; kk++) {
+        loadFrags(cur, kk + 1, fa[(kk + 1) & 1], fb[(kk + 1) & 1]);
+        mfmaStep(fa[kk & 1], fb[kk & 1]);
+      }
+      if (i + 1 < nk) {
+        // all of this wavefront's reads of slab i are in registers; slab i+1
+        // has landed for this wavefront; then wait for the other wavefronts
+        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(
+                         kInFlight)
+                     : "memory");
+        issue(ktBegin + i + NS, cur);
+        loadFrags((i + 1) % NS, 0, fa[0], fb[0]);
+      }
+      mfmaStep(fa[(KSTEPS - 1) & 1], fb[(KSTEPS - 1) & 1]);
+    }
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // no DMA may outlive the loop
+
+  if (numSlices > 1) {
+    storePartial<MI, NI, THREADS>(p, acc, tile, slice, numSlices, tid);
+    return;
+  }
+  epilogueStore<MI, NI, WTM, WTN, EPI, 8>(p, acc, m0, n0, waveM, waveN, lane);
+#endif
+}
+
+// ================================================================== staged ==
 // VEC == 8: N, K multiples of 8 and 16-byte aligned operands (128-bit global
 // accesses).  VEC == 1: any shape/alignment, scalar global accesses.
 template <int BM, int BN, int BK, int WM, int WN, int EPI, bool B_NK, int VEC>
-__global__ __launch_bounds__(WM *WN *kWave) void gemmKernel(GemmParams p) {
+__global__ __launch_bounds__(WM *WN *kWave) void gemmStagedKernel(GemmParams p) {
   constexpr int kThreads = WM * WN * kWave;
-  constexpr int WTM = BM / WM, WTN = BN / WN; // wavefront tile
-  constexpr int MI = WTM / 32, NI = WTN / 32; // 32x32 MFMA blocks per wave
+  constexpr int WTM = BM / WM, WTN = BN / WN;
+  constexpr int MI = WTM / 32, NI = WTN / 32;
   static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile must be 32-aligned");
   static_assert(BK % 16 == 0, "BK must be a multiple of the MFMA k (16)");
-  constexpr int A_LD = BK + 8;     // halves per LDS row of A (and of B when NK)
-  constexpr int BP_LD = BN + 8;    // dwords per LDS row of k-pair-packed B
+  constexpr int A_LD = BK + 8;  // halves per LDS row of A (and of B when NK)
+  constexpr int BP_LD = BN + 8; // dwords per LDS row of k-pair-packed B
   constexpr int A_BYTES = BM * A_LD * 2;
   constexpr int B_BYTES = B_NK ? BN * A_LD * 2 : (BK / 2) * BP_LD * 4;
   constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
 
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
 
   const int tid = threadIdx.x;
   const int lane = tid % kWave;
   const int wave = tid / kWave;
   const int waveM = wave / WN, waveN = wave % WN;
 
-  // ---- tile assignment (XCD-contiguous) ----
   const int nTiles = p.tilesM * p.tilesN;
-  int tile;
-  {
-    const int pid = blockIdx.x;
-    const int q = nTiles / kNumXcd, r = nTiles % kNumXcd;
-    const int xcd = pid % kNumXcd, loc = pid / kNumXcd;
-    tile = xcd * q + (xcd < r ? xcd : r) + loc;
-  }
-  const int tileM = tile / p.tilesN, tileN = tile % p.tilesN;
+  const int tile = tileForBlock(nTiles);
+  int tileM, tileN;
+  tileCoords(tile, p.tilesM, p.tilesN, &tileM, &tileN);
   const int m0 = tileM * BM, n0 = tileN * BN;
   const int slice = blockIdx.y, numSlices = gridDim.y;
 
@@ -127,13 +531,12 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmKernel(GemmParams p) {
       for (int e = 0; e < 16; e++)
         acc[i][j][e] = 0.f;
 
-  // ---- global -> register staging ----
-  constexpr int A_VECS = BM * BK / 8;                 // 16-byte vectors of A
+  constexpr int A_VECS = BM * BK / 8;
   constexpr int A_PER_T = (A_VECS + kThreads - 1) / kThreads;
-  constexpr int A_VPR = BK / 8;                       // vectors per A row
+  constexpr int A_VPR = BK / 8;
   constexpr int BNK_VECS = BN * BK / 8;
   constexpr int BNK_PER_T = (BNK_VECS + kThreads - 1) / kThreads;
-  constexpr int BKN_ITEMS = (BK / 2) * (BN / 8);      // (k-pair, 8 columns)
+  constexpr int BKN_ITEMS = (BK / 2) * (BN / 8); // (k-pair, 8 columns)
   constexpr int BKN_PER_T = (BKN_ITEMS + kThreads - 1) / kThreads;
   constexpr int BKN_CPR = BN / 8;
 
@@ -314,7 +717,6 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmKernel(GemmParams p) {
     }
   };
 
-  // ---- main loop ----
   if (ktBegin < ktEnd) {
     if (VEC == 8) {
       loadGlobal(ktBegin);
@@ -341,126 +743,23 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmKernel(GemmParams p) {
     }
   }
 
-  // ---- split-K: exchange partial tiles, last arrival reduces ----
   if (numSlices > 1) {
-    __shared__ uint32_t sArrival;
-    constexpr int ACC_V4 = MI * NI * 4; // float4 vectors per thread
-    float4v *ws = reinterpret_cast<float4v *>(p.workspace) +
-                  (int64_t(tile) * numSlices) * (ACC_V4 * kThreads);
-    {
-      float4v *mine = ws + int64_t(slice) * (ACC_V4 * kThreads);
-#pragma unroll
-      for (int i = 0; i < MI; i++)
-#pragma unroll
-        for (int j = 0; j < NI; j++)
-#pragma unroll
-          for (int g = 0; g < 4; g++) {
-            float4v v;
-#pragma unroll
-            for (int e = 0; e < 4; e++)
-              v[e] = acc[i][j][g * 4 + e];
-            mine[((i * NI + j) * 4 + g) * kThreads + tid] = v;
-          }
-    }
-    __threadfence();
-    __syncthreads();
-    if (tid == 0)
-      sArrival = __hip_atomic_fetch_add(&p.counters[tile], 1u,
-                                        __ATOMIC_ACQ_REL,
-                                        __HIP_MEMORY_SCOPE_AGENT);
-    __syncthreads();
-    if (sArrival != uint32_t(numSlices - 1))
-      return; // uniform across the workgroup
-    __threadfence();
-#pragma unroll
-    for (int i = 0; i < MI; i++)
-#pragma unroll
-      for (int j = 0; j < NI; j++)
-#pragma unroll
-        for (int e = 0; e < 16; e++)
-          acc[i][j][e] = 0.f;
-    for (int s = 0; s < numSlices; s++) {
-      const float4v *part = ws + int64_t(s) * (ACC_V4 * kThreads);
-#pragma unroll
-      for (int i = 0; i < MI; i++)
-#pragma unroll
-        for (int j = 0; j < NI; j++)
-#pragma unroll
-          for (int g = 0; g < 4; g++) {
-            const float4v v = __builtin_nontemporal_load(
-                &part[((i * NI + j) * 4 + g) * kThreads + tid]);
-#pragma unroll
-            for (int e = 0; e < 4; e++)
-              acc[i][j][g * 4 + e] += v[e];
-          }
-    }
-    if (tid == 0)
-      __hip_atomic_store(&p.counters[tile], 0u, __ATOMIC_RELAXED,
-                         __HIP_MEMORY_SCOPE_AGENT);
+    storePartial<MI, NI, kThreads>(p, acc, tile, slice, numSlices, tid);
+    return;
   }
-
-  // ---- epilogue ----
-  // Transposed MFMA block: accumulator e of lane l is
-  //   column n = 8*(e/4) + 4*(l/32) + e%4,  row m = l%32   (within the block).
-  const int l32 = lane % 32, kb = lane / 32;
-  const bool useC = p.beta != 0.f;
-#pragma unroll
-  for (int i = 0; i < MI; i++) {
-    const int m = m0 + waveM * WTM + i * 32 + l32;
-    if (m >= p.M)
-      continue;
-    const int64_t cRow = int64_t(m % p.cRowPeriod) * p.ldc;
-    const int64_t dRow = int64_t(m) * p.ldd;
-#pragma unroll
-    for (int j = 0; j < NI; j++) {
-#pragma unroll
-      for (int g = 0; g < 4; g++) {
-        const int n = n0 + waveN * WTN + j * 32 + g * 8 + kb * 4;
-        if (VEC == 8) {
-          if (n >= p.N)
-            continue;
-          float c[4] = {0.f, 0.f, 0.f, 0.f};
-          if (useC) {
-            const half4 cv = *reinterpret_cast<const half4 *>(p.C + cRow + n);
-#pragma unroll
-            for (int e = 0; e < 4; e++)
-              c[e] = float(cv[e]);
-          }
-          half4 o;
-#pragma unroll
-          for (int e = 0; e < 4; e++) {
-            float v = p.alpha * acc[i][j][g * 4 + e];
-            if (useC)
-              v += p.beta * c[e];
-            o[e] = _Float16(activate<EPI>(v));
-          }
-          *reinterpret_cast<half4 *>(p.D + dRow + n) = o;
-        } else {
-#pragma unroll
-          for (int e = 0; e < 4; e++) {
-            if (n + e < p.N) {
-              float v = p.alpha * acc[i][j][g * 4 + e];
-              if (useC)
-                v += p.beta * float(p.C[cRow + n + e]);
-              p.D[dRow + n + e] = _Float16(activate<EPI>(v));
-            }
-          }
-        }
-      }
-    }
-  }
+  epilogueStore<MI, NI, WTM, WTN, EPI, VEC>(p, acc, m0, n0, waveM, waveN, lane);
 }
 
 // ------------------------------------------------------------ kernel table --
-template <int BM, int BN, int BK, int WM, int WN, int EPI, bool B_NK, int VEC>
-Status launchInstance(const GemmProblem &pr, hipStream_t s) {
-  constexpr int kThreads = WM * WN * kWave;
-  constexpr int A_LD = BK + 8, BP_LD = BN + 8;
-  constexpr int A_BYTES = BM * A_LD * 2;
-  constexpr int B_BYTES = B_NK ? BN * A_LD * 2 : (BK / 2) * BP_LD * 4;
-  constexpr int SMEM = 2 * (A_BYTES + B_BYTES);
-
+struct LaunchPlan {
   GemmParams p;
+  int splitK;
+  int64_t nTiles;
+};
+
+template <int BM, int BN, int BK>
+Status planLaunch(const GemmProblem &pr, LaunchPlan *plan) {
+  GemmParams &p = plan->p;
   p.A = pr.A;
   p.B = pr.B;
   p.C = pr.C;
@@ -482,39 +781,96 @@ Status launchInstance(const GemmProblem &pr, hipStream_t s) {
   if (splitK > kTiles)
     splitK = kTiles > 0 ? kTiles : 1;
   p.kTilesPerSlice = (kTiles + splitK - 1) / splitK;
-  // Drop slices that would be empty after rounding up.
-  if (p.kTilesPerSlice > 0)
+  if (p.kTilesPerSlice > 0) // drop slices that rounding up left empty
     splitK = (kTiles + p.kTilesPerSlice - 1) / p.kTilesPerSlice;
   if (splitK < 1)
     splitK = 1;
-  const int64_t nTiles = int64_t(p.tilesM) * p.tilesN;
-  HOM_CHECK_RET(nTiles < (int64_t(1) << 30), Status::kInvalidArgument,
-                "gemm: too many output tiles (%lld)", (long long)nTiles);
+  plan->splitK = splitK;
+  plan->nTiles = int64_t(p.tilesM) * p.tilesN;
+  HOM_CHECK_RET(plan->nTiles < (int64_t(1) << 30), Status::kInvalidArgument,
+                "gemm: too many output tiles (%lld)", (long long)plan->nTiles);
   p.workspace = nullptr;
-  p.counters = nullptr;
   if (splitK > 1) {
     const size_t wsBytes =
-        size_t(nTiles) * splitK * size_t(BM) * BN * sizeof(float);
+        size_t(plan->nTiles) * splitK * size_t(BM) * BN * sizeof(float);
     p.workspace = static_cast<float *>(scratch(kWorkspace, wsBytes, false));
-    p.counters = static_cast<uint32_t *>(
-        scratch(kCounters, size_t(nTiles) * sizeof(uint32_t), true));
-    if (!p.workspace || !p.counters)
+    if (!p.workspace)
       return Status::kInternal;
   }
-  auto kernel = gemmKernel<BM, BN, BK, WM, WN, EPI, B_NK, VEC>;
-  static bool attrSet = false;
-  if (!attrSet && SMEM > 48 * 1024) {
+  return Status::kSuccess;
+}
+
+template <typename K> Status allowLds(K kernel, int bytes, bool *done) {
+  if (!*done && bytes > 48 * 1024) {
     HOM_HIP_RET(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                     hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    SMEM),
+                                    bytes),
                 Status::kInternal);
   }
-  attrSet = true;
-  if (nTiles == 0)
-    return Status::kSuccess;
-  kernel<<<dim3((unsigned)nTiles, (unsigned)splitK), dim3(kThreads), SMEM, s>>>(
-      p);
+  *done = true;
+  return Status::kSuccess;
+}
+
+template <int BM, int BN, int WM, int WN, int EPI, int VEC>
+Status launchReduce(const LaunchPlan &plan, hipStream_t s) {
+  splitKReduceKernel<BM, BN, WM, WN, EPI, VEC>
+      <<<dim3((unsigned)plan.nTiles), dim3(WM * WN * kWave), 0, s>>>(
+          plan.p, plan.splitK);
   HOM_HIP_RET(hipGetLastError(), Status::kInternal);
+  return Status::kSuccess;
+}
+
+template <int BM, int BN, int BK, int WM, int WN, int EPI, bool B_NK, int VEC>
+Status launchStaged(const GemmProblem &pr, hipStream_t s) {
+  constexpr int A_LD = BK + 8, BP_LD = BN + 8;
+  constexpr int A_BYTES = BM * A_LD * 2;
+  constexpr int B_BYTES = B_NK ? BN * A_LD * 2 : (BK / 2) * BP_LD * 4;
+  constexpr int SMEM = 2 * (A_BYTES + B_BYTES);
+  LaunchPlan plan;
+  Status st = planLaunch<BM, BN, BK>(pr, &plan);
+  if (st != Status::kSuccess)
+    return st;
+  auto kernel = gemmStagedKernel<BM, BN, BK, WM, WN, EPI, B_NK, VEC>;
+  static bool attrSet = false;
+  st = allowLds(kernel, SMEM, &attrSet);
+  if (st != Status::kSuccess)
+    return st;
+  if (plan.nTiles == 0)
+    return Status::kSuccess;
+  kernel<<<dim3((unsigned)plan.nTiles, (unsigned)plan.splitK),
+           dim3(WM * WN * kWave), SMEM, s>>>(plan.p);
+  HOM_HIP_RET(hipGetLastError(), Status::kInternal);
+  if (plan.splitK > 1)
+    return launchReduce<BM, BN, WM, WN, EPI, VEC>(plan, s);
+  return Status::kSuccess;
+}
+
+template <int BM, int BN, int WM, int WN, int NS, int EPI, bool B_NK>
+Status launchDma(const GemmProblem &pr, hipStream_t s) {
+  constexpr int SMEM = NS * (BM + BN) * 64 * 2;
+  LaunchPlan plan;
+  Status st = planLaunch<BM, BN, 64>(pr, &plan);
+  if (st != Status::kSuccess)
+    return st;
+  // 32-bit DMA offsets: a row-major B slab is addressed from the matrix base.
+  HOM_CHECK_RET(B_NK || pr.K * pr.ldb * 2 < (int64_t(1) << 31),
+                Status::kInvalidArgument,
+                "gemm: B larger than 2 GiB is not supported by this kernel");
+  HOM_CHECK_RET(int64_t(BM) * pr.lda * 2 < (int64_t(1) << 31) &&
+                    int64_t(BN) * pr.ldb * 2 < (int64_t(1) << 31),
+                Status::kInvalidArgument, "gemm: leading dimension too large");
+  auto kernel = gemmDmaKernel<BM, BN, WM, WN, NS, EPI, B_NK>;
+  static bool attrSet = false;
+  st = allowLds(kernel, SMEM, &attrSet);
+  if (st != Status::kSuccess)
+    return st;
+  if (plan.nTiles == 0)
+    return Status::kSuccess;
+  kernel<<<dim3((unsigned)plan.nTiles, (unsigned)plan.splitK),
+           dim3(WM * WN * kWave), SMEM, s>>>(plan.p);
+  HOM_HIP_RET(hipGetLastError(), Status::kInternal);
+  if (plan.splitK > 1)
+    return launchReduce<BM, BN, WM, WN, EPI, 8>(plan, s);
   return Status::kSuccess;
 }
 
@@ -526,33 +882,57 @@ struct KernelEntry {
   LaunchFn nt; // B as [N, K]
 };
 
-#define HOM_GEMM_ENTRY(BM, BN, BK, WM, WN, EPI_ENUM, EPI_STR, ACT, VEC)        \
+// Names follow the reference generator's scheme (python/hom_manifest.py:56-74):
+// <arch>_<opclass>_<acc><instr>gemm_<type>_<tile>_<K>x<stages>_<warps>_<layout>_
+// align<n>_<epilogue>; "linear"/"gelu" in the name is what activation is derived
+// from (GemmRunner.h:200-206).
+#define HOM_DMA_ENTRY(BM, BN, WM, WN, NS, EPI_ENUM, EPI_STR, ACT)              \
+  {                                                                            \
+    {"hom_gfx950_mfma_f16_s32x32x16gemm_f16_" #BM "x" #BN "_64x" #NS "_w" #WM  \
+     "x" #WN "_nn_align8_" EPI_STR,                                            \
+     BM, BN, 64, WM, WN, 8, ACT, EPI_ENUM},                                    \
+        launchDma<BM, BN, WM, WN, NS, int(EPI_ENUM), false>,                   \
+        launchDma<BM, BN, WM, WN, NS, int(EPI_ENUM), true>                     \
+  }
+#define HOM_DMA_TILE(BM, BN, WM, WN, NS)                                       \
+  HOM_DMA_ENTRY(BM, BN, WM, WN, NS, Epilogue::kLinear, "linear", 0),           \
+      HOM_DMA_ENTRY(BM, BN, WM, WN, NS, Epilogue::kGeluErf, "gelu", 1),        \
+      HOM_DMA_ENTRY(BM, BN, WM, WN, NS, Epilogue::kGeluTanh, "gelutanh", 1)
+
+#define HOM_STAGED_ENTRY(BM, BN, BK, WM, WN, EPI_ENUM, EPI_STR, ACT, VEC)      \
   {                                                                            \
     {"hom_gfx950_mfma_f16_s32x32x16gemm_f16_" #BM "x" #BN "_" #BK "x2_w" #WM   \
      "x" #WN "_nn_align" #VEC "_" EPI_STR,                                     \
      BM, BN, BK, WM, WN, VEC, ACT, EPI_ENUM},                                  \
-        launchInstance<BM, BN, BK, WM, WN, int(EPI_ENUM), false, VEC>,         \
-        launchInstance<BM, BN, BK, WM, WN, int(EPI_ENUM), true, VEC>           \
+        launchStaged<BM, BN, BK, WM, WN, int(EPI_ENUM), false, VEC>,           \
+        launchStaged<BM, BN, BK, WM, WN, int(EPI_ENUM), true, VEC>             \
   }
-
-#define HOM_GEMM_TILE(BM, BN, BK, WM, WN, VEC)                                 \
-  HOM_GEMM_ENTRY(BM, BN, BK, WM, WN, Epilogue::kLinear, "linear", 0, VEC),     \
-      HOM_GEMM_ENTRY(BM, BN, BK, WM, WN, Epilogue::kGeluErf, "gelu", 1, VEC),  \
-      HOM_GEMM_ENTRY(BM, BN, BK, WM, WN, Epilogue::kGeluTanh, "gelutanh", 1,   \
-                     VEC)
+#define HOM_STAGED_TILE(BM, BN, BK, WM, WN, VEC)                               \
+  HOM_STAGED_ENTRY(BM, BN, BK, WM, WN, Epilogue::kLinear, "linear", 0, VEC),   \
+      HOM_STAGED_ENTRY(BM, BN, BK, WM, WN, Epilogue::kGeluErf, "gelu", 1,      \
+                       VEC),                                                   \
+      HOM_STAGED_ENTRY(BM, BN, BK, WM, WN, Epilogue::kGeluTanh, "gelutanh", 1, \
+                       VEC)
 
 // Manifest order is part of the ABI: compiled modules carry indices into it.
 // Append new entries at the end.
 const KernelEntry kKernels[] = {
-    HOM_GEMM_TILE(128, 128, 32, 2, 2, 8),
-    HOM_GEMM_TILE(64, 64, 32, 2, 2, 8),
-    HOM_GEMM_TILE(128, 64, 32, 2, 2, 8),
-    HOM_GEMM_TILE(64, 128, 32, 2, 2, 8),
-    HOM_GEMM_TILE(256, 128, 32, 2, 2, 8),
-    HOM_GEMM_TILE(128, 256, 32, 2, 2, 8),
-    HOM_GEMM_TILE(128, 128, 64, 2, 2, 8),
-    HOM_GEMM_TILE(64, 64, 64, 2, 2, 8),
-    HOM_GEMM_TILE(64, 64, 32, 2, 2, 1),
+    HOM_DMA_TILE(128, 128, 2, 2, 4),
+    HOM_DMA_TILE(64, 64, 2, 2, 4),
+    HOM_DMA_TILE(128, 64, 2, 2, 4),
+    HOM_DMA_TILE(64, 128, 2, 2, 4),
+    HOM_DMA_TILE(256, 128, 2, 2, 3),
+    HOM_DMA_TILE(128, 256, 2, 2, 3),
+    HOM_DMA_TILE(256, 256, 2, 2, 2),
+    HOM_DMA_TILE(128, 128, 2, 2, 2),
+    HOM_DMA_TILE(64, 64, 2, 2, 8),
+    HOM_DMA_TILE(128, 128, 2, 4, 4),
+    HOM_DMA_TILE(256, 128, 4, 2, 3),
+    HOM_DMA_TILE(256, 256, 2, 4, 2),
+    HOM_DMA_TILE(128, 256, 2, 4, 3),
+    HOM_STAGED_TILE(128, 128, 32, 2, 2, 8),
+    HOM_STAGED_TILE(64, 64, 64, 2, 2, 8),
+    HOM_STAGED_TILE(64, 64, 32, 2, 2, 1),
 };
 constexpr int kNumKernels = sizeof(kKernels) / sizeof(kKernels[0]);
 

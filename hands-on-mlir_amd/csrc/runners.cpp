@@ -281,6 +281,18 @@ Status runGemmNvte(int64_t rankA, void *dstA, bool transa, int64_t rankB,
              &sel, &sk);
   int idx = int(sel);
   pr.splitK = sk;
+  // Profiling knob: HOM_NVTE_GEMM_KERNEL="<manifest name>[,<splitK>]" pins the
+  // kernel used on this path (the epilogue must match the activation).
+  if (const char *force = getenv("HOM_NVTE_GEMM_KERNEL")) {
+    std::string f(force);
+    const size_t comma = f.find(',');
+    const std::string name = f.substr(0, comma);
+    for (int i = 0; i < gemmKernelCount(); i++)
+      if (name == gemmKernelInfo(i).name && gemmKernelInfo(i).epilogue == epi) {
+        idx = i;
+        pr.splitK = comma == std::string::npos ? 1 : atoi(f.c_str() + comma + 1);
+      }
+  }
   if (gemmKernelInfo(idx).alignment == 8 && alignmentClass(pr) != 8) {
     idx = findKernel(64, 64, 32, epi, 1);
     pr.splitK = 1;

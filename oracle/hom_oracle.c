@@ -154,20 +154,20 @@ static double activate(double v, int act) {
 /* ---------------------------------------------------------------- GEMM --- */
 
 /* D[m,n] = act(alpha * sum_k A[m,k] B(k,n) + beta * C[(m % c_row_period), n])
- * A [M,K] row-major fp16; B [K,N] row-major, or [N,K] when b_is_nk;
- * C fp16 with leading dimension ldc (ignored when beta == 0);
+ * A [M,K] row-major; B [K,N] row-major, or [N,K] when b_is_nk; C with leading
+ * dimension ldc (ignored when beta == 0);
  * act: 0 linear, 1 GELU erf, 2 GELU tanh, 3 GELU polynomial.
- * Output D as float (not rounded). */
-ORACLE_API void hom_oracle_gemm(const uint16_t *A, const uint16_t *B,
-                                const uint16_t *C, float *D, int64_t M,
-                                int64_t N, int64_t K, int64_t ldc,
-                                int64_t c_row_period, float alpha, float beta,
-                                int act, int b_is_nk) {
+ * Inputs are float (fp16 values converted exactly); output D float, unrounded. */
+ORACLE_API void hom_oracle_gemm_f32in(const float *A, const float *B,
+                                      const float *C, float *D, int64_t M,
+                                      int64_t N, int64_t K, int64_t ldc,
+                                      int64_t c_row_period, float alpha,
+                                      float beta, int act, int b_is_nk) {
   /* B as doubles, K x N, so the inner loop streams */
   double *Bd = (double *)malloc(sizeof(double) * (size_t)(K * N > 0 ? K * N : 1));
   for (int64_t k = 0; k < K; k++)
     for (int64_t n = 0; n < N; n++)
-      Bd[k * N + n] = b_is_nk ? h2d(B[n * K + k]) : h2d(B[k * N + n]);
+      Bd[k * N + n] = b_is_nk ? (double)B[n * K + k] : (double)B[k * N + n];
   if (c_row_period < 1)
     c_row_period = 1;
 #pragma omp parallel
@@ -178,7 +178,7 @@ ORACLE_API void hom_oracle_gemm(const uint16_t *A, const uint16_t *B,
       for (int64_t n = 0; n < N; n++)
         acc[n] = 0.0;
       for (int64_t k = 0; k < K; k++) {
-        const double a = h2d(A[m * K + k]);
+        const double a = (double)A[m * K + k];
         const double *brow = Bd + k * N;
         for (int64_t n = 0; n < N; n++)
           acc[n] += a * brow[n];
@@ -186,7 +186,7 @@ ORACLE_API void hom_oracle_gemm(const uint16_t *A, const uint16_t *B,
       for (int64_t n = 0; n < N; n++) {
         double v = (double)alpha * acc[n];
         if (beta != 0.0f)
-          v += (double)beta * h2d(C[(m % c_row_period) * ldc + n]);
+          v += (double)beta * (double)C[(m % c_row_period) * ldc + n];
         D[m * N + n] = (float)activate(v, act);
       }
     }
@@ -195,45 +195,88 @@ ORACLE_API void hom_oracle_gemm(const uint16_t *A, const uint16_t *B,
   free(Bd);
 }
 
+static float *halves_to_floats(const uint16_t *h, int64_t n) {
+  if (!h)
+    return NULL;
+  float *f = (float *)malloc(sizeof(float) * (size_t)(n > 0 ? n : 1));
+  for (int64_t i = 0; i < n; i++)
+    f[i] = hom_oracle_half_to_float(h[i]);
+  return f;
+}
+
+/* Same with fp16 operands (bit patterns). */
+ORACLE_API void hom_oracle_gemm(const uint16_t *A, const uint16_t *B,
+                                const uint16_t *C, float *D, int64_t M,
+                                int64_t N, int64_t K, int64_t ldc,
+                                int64_t c_row_period, float alpha, float beta,
+                                int act, int b_is_nk) {
+  if (c_row_period < 1)
+    c_row_period = 1;
+  float *a = halves_to_floats(A, M * K), *b = halves_to_floats(B, K * N);
+  float *c = beta != 0.0f ? halves_to_floats(C, (c_row_period - 1) * ldc + N)
+                          : NULL;
+  hom_oracle_gemm_f32in(a, b, c, D, M, N, K, ldc, c_row_period, alpha, beta, act,
+                        b_is_nk);
+  free(a);
+  free(b);
+  free(c);
+}
+
 /* ----------------------------------------------------------- LayerNorm --- */
 
 /* out[r,:] = (v - mean(v)) / sqrt(var(v) + eps) * gamma + beta with
- * v = x[r,:] (+ res[r,:]); biased variance.  res/gamma/beta may be NULL. */
-ORACLE_API void hom_oracle_layernorm_f16(const uint16_t *x, const uint16_t *res,
-                                         const uint16_t *gamma,
-                                         const uint16_t *beta, float *out,
-                                         int64_t rows, int64_t hidden,
-                                         float eps) {
+ * v = x[r,:] (+ res[r,:]); biased variance.  res/gamma/beta may be NULL.
+ * out may alias x. */
+ORACLE_API void hom_oracle_layernorm_f32in(const float *x, const float *res,
+                                           const float *gamma,
+                                           const float *beta, float *out,
+                                           int64_t rows, int64_t hidden,
+                                           float eps) {
 #pragma omp parallel for schedule(static)
   for (int64_t r = 0; r < rows; r++) {
     double sum = 0.0;
     for (int64_t j = 0; j < hidden; j++) {
-      double v = h2d(x[r * hidden + j]);
+      double v = x[r * hidden + j];
       if (res)
-        v += h2d(res[r * hidden + j]);
+        v += res[r * hidden + j];
       sum += v;
     }
     const double mean = sum / (double)hidden;
     double sq = 0.0;
     for (int64_t j = 0; j < hidden; j++) {
-      double v = h2d(x[r * hidden + j]);
+      double v = x[r * hidden + j];
       if (res)
-        v += h2d(res[r * hidden + j]);
+        v += res[r * hidden + j];
       sq += (v - mean) * (v - mean);
     }
     const double rstd = 1.0 / sqrt(sq / (double)hidden + (double)eps);
     for (int64_t j = 0; j < hidden; j++) {
-      double v = h2d(x[r * hidden + j]);
+      double v = x[r * hidden + j];
       if (res)
-        v += h2d(res[r * hidden + j]);
+        v += res[r * hidden + j];
       double y = (v - mean) * rstd;
       if (gamma)
-        y *= h2d(gamma[j]);
+        y *= gamma[j];
       if (beta)
-        y += h2d(beta[j]);
+        y += beta[j];
       out[r * hidden + j] = (float)y;
     }
   }
+}
+
+ORACLE_API void hom_oracle_layernorm_f16(const uint16_t *x, const uint16_t *res,
+                                         const uint16_t *gamma,
+                                         const uint16_t *beta, float *out,
+                                         int64_t rows, int64_t hidden,
+                                         float eps) {
+  float *xf = halves_to_floats(x, rows * hidden),
+        *rf = halves_to_floats(res, rows * hidden),
+        *gf = halves_to_floats(gamma, hidden), *bf = halves_to_floats(beta, hidden);
+  hom_oracle_layernorm_f32in(xf, rf, gf, bf, out, rows, hidden, eps);
+  free(xf);
+  free(rf);
+  free(gf);
+  free(bf);
 }
 
 ORACLE_API void hom_oracle_layernorm_f32(const float *x, float *out,
@@ -273,9 +316,10 @@ ORACLE_API void hom_oracle_row_stats(const float *d, float *var, float *mean,
 
 /* qkv [bs, seq, 3, heads, d] fp16; cu int32[bs+1]; out [bs, seq, heads, d]
  * float.  Keys >= len_b are masked; query rows >= len_b produce zeros. */
-ORACLE_API void hom_oracle_attention(const uint16_t *qkv, const int32_t *cu,
-                                     float *out, int64_t bs, int64_t seq,
-                                     int64_t heads, int64_t d, float scale) {
+ORACLE_API void hom_oracle_attention_f32in(const float *qkv, const int32_t *cu,
+                                           float *out, int64_t bs, int64_t seq,
+                                           int64_t heads, int64_t d,
+                                           float scale) {
   const int64_t tok = 3 * heads * d;
 #pragma omp parallel
   {
@@ -288,7 +332,7 @@ ORACLE_API void hom_oracle_attention(const uint16_t *qkv, const int32_t *cu,
           len = 0;
         if (len > seq)
           len = seq;
-        const uint16_t *base = qkv + b * seq * tok;
+        const float *base = qkv + b * seq * tok;
         for (int64_t q = 0; q < seq; q++) {
           float *o = out + ((b * seq + q) * heads + h) * d;
           if (q >= len) {
@@ -296,13 +340,13 @@ ORACLE_API void hom_oracle_attention(const uint16_t *qkv, const int32_t *cu,
               o[j] = 0.0f;
             continue;
           }
-          const uint16_t *qv = base + q * tok + h * d;
+          const float *qv = base + q * tok + h * d;
           double mx = -INFINITY;
           for (int64_t k = 0; k < len; k++) {
-            const uint16_t *kv = base + k * tok + (heads + h) * d;
+            const float *kv = base + k * tok + (heads + h) * d;
             double s = 0.0;
             for (int64_t j = 0; j < d; j++)
-              s += h2d(qv[j]) * h2d(kv[j]);
+              s += (double)qv[j] * (double)kv[j];
             p[k] = s * (double)scale;
             if (p[k] > mx)
               mx = p[k];
@@ -315,7 +359,7 @@ ORACLE_API void hom_oracle_attention(const uint16_t *qkv, const int32_t *cu,
           for (int64_t j = 0; j < d; j++) {
             double acc = 0.0;
             for (int64_t k = 0; k < len; k++)
-              acc += p[k] * h2d(base[k * tok + (2 * heads + h) * d + j]);
+              acc += p[k] * (double)base[k * tok + (2 * heads + h) * d + j];
             o[j] = (float)(acc / denom);
           }
         }
@@ -323,6 +367,14 @@ ORACLE_API void hom_oracle_attention(const uint16_t *qkv, const int32_t *cu,
     }
     free(p);
   }
+}
+
+ORACLE_API void hom_oracle_attention(const uint16_t *qkv, const int32_t *cu,
+                                     float *out, int64_t bs, int64_t seq,
+                                     int64_t heads, int64_t d, float scale) {
+  float *f = halves_to_floats(qkv, bs * seq * 3 * heads * d);
+  hom_oracle_attention_f32in(f, cu, out, bs, seq, heads, d, scale);
+  free(f);
 }
 
 /* ---------------------------------------------------------- cu_seqlens --- */
@@ -418,57 +470,66 @@ ORACLE_API void hom_oracle_gather(const int64_t *indices, const void *value,
 
 /* -------------------------------------------------------- BERT encoder --- */
 
-static void round_to_half(const float *src, uint16_t *dst, int64_t n) {
+/* Round every value to fp16 and back (what storing the tensor as fp16 does). */
+static void round_through_half(float *x, int64_t n) {
 #pragma omp parallel for schedule(static)
   for (int64_t i = 0; i < n; i++)
-    dst[i] = hom_oracle_float_to_half(src[i]);
+    x[i] = hom_oracle_half_to_float(hom_oracle_float_to_half(x[i]));
 }
 
-/* The lowered encoder's call list with fp16 rounding wherever the GPU path
- * stores fp16.  Weights per layer: Wqkv [H,3H], Wo [H,H], W1 [H,F], W2 [F,H]
- * (row-major [K,N]), concatenated layer after layer in that order.
- * h: in/out hidden states [rows = bs*seq, H] as fp16 (updated in place).
- * gelu_act: 1 erf, 2 tanh.  out_f32 (may be NULL) receives the final layer
- * norm before its rounding to fp16. */
-ORACLE_API void hom_oracle_bert_encoder(uint16_t *h, const uint16_t *weights,
+/* The lowered encoder's call list.  Weights per layer: Wqkv [H,3H], Wo [H,H],
+ * W1 [H,F], W2 [F,H] (row-major [K,N]), concatenated layer after layer in that
+ * order, fp16.  h: in/out hidden states [rows = bs*seq, H] as float holding
+ * fp16-representable values on entry.
+ * round_intermediates != 0: every tensor the GPU path stores as fp16 is rounded
+ * to fp16 here too (the fp16-boundary-faithful oracle); == 0: intermediates
+ * stay unrounded (the pure fp32 reference of the same fp16 weights/inputs).
+ * gelu_act: 1 erf, 2 tanh.  On return h holds the final layer norm (rounded
+ * only if round_intermediates). */
+ORACLE_API void hom_oracle_bert_encoder(float *h, const uint16_t *weights,
                                         const int32_t *cu, int64_t layers,
                                         int64_t bs, int64_t seq, int64_t hidden,
                                         int64_t heads, int64_t ffn, float eps,
-                                        int gelu_act, float *out_f32) {
+                                        int gelu_act, int round_intermediates) {
   const int64_t rows = bs * seq, d = hidden / heads;
-  const int64_t maxw = 3 * hidden > ffn ? 3 * hidden : ffn;
-  float *tmp = (float *)malloc(sizeof(float) * (size_t)(rows * maxw));
-  uint16_t *qkv = (uint16_t *)malloc(2 * (size_t)(rows * 3 * hidden));
-  uint16_t *attn = (uint16_t *)malloc(2 * (size_t)(rows * hidden));
-  uint16_t *f = (uint16_t *)malloc(2 * (size_t)(rows * ffn));
+  float *qkv = (float *)malloc(sizeof(float) * (size_t)(rows * 3 * hidden));
+  float *attn = (float *)malloc(sizeof(float) * (size_t)(rows * hidden));
+  float *f = (float *)malloc(sizeof(float) * (size_t)(rows * ffn));
   const float scale = (float)(1.0 / sqrt((double)d));
+  const int r = round_intermediates;
   const uint16_t *w = weights;
   for (int64_t l = 0; l < layers; l++) {
-    const uint16_t *wqkv = w, *wo = wqkv + hidden * 3 * hidden,
-                   *w1 = wo + hidden * hidden, *w2 = w1 + hidden * ffn;
-    w = w2 + ffn * hidden;
-    hom_oracle_gemm(h, wqkv, NULL, tmp, rows, 3 * hidden, hidden, 0, 1, 1.0f,
-                    0.0f, 0, 0);
-    round_to_half(tmp, qkv, rows * 3 * hidden);
-    hom_oracle_attention(qkv, cu, tmp, bs, seq, heads, d, scale);
-    round_to_half(tmp, attn, rows * hidden);
-    hom_oracle_gemm(attn, wo, h, tmp, rows, hidden, hidden, hidden, rows, 1.0f,
-                    1.0f, 0, 0);
-    round_to_half(tmp, h, rows * hidden);
-    hom_oracle_layernorm_f16(h, NULL, NULL, NULL, tmp, rows, hidden, eps);
-    round_to_half(tmp, h, rows * hidden);
-    hom_oracle_gemm(h, w1, NULL, tmp, rows, ffn, hidden, 0, 1, 1.0f, 0.0f,
-                    gelu_act, 0);
-    round_to_half(tmp, f, rows * ffn);
-    hom_oracle_gemm(f, w2, h, tmp, rows, hidden, ffn, hidden, rows, 1.0f, 1.0f,
-                    0, 0);
-    round_to_half(tmp, h, rows * hidden);
-    hom_oracle_layernorm_f16(h, NULL, NULL, NULL, tmp, rows, hidden, eps);
-    if (out_f32 && l == layers - 1)
-      memcpy(out_f32, tmp, sizeof(float) * (size_t)(rows * hidden));
-    round_to_half(tmp, h, rows * hidden);
+    float *wqkv = halves_to_floats(w, hidden * 3 * hidden);
+    w += hidden * 3 * hidden;
+    float *wo = halves_to_floats(w, hidden * hidden);
+    w += hidden * hidden;
+    float *w1 = halves_to_floats(w, hidden * ffn);
+    w += hidden * ffn;
+    float *w2 = halves_to_floats(w, ffn * hidden);
+    w += ffn * hidden;
+    hom_oracle_gemm_f32in(h, wqkv, NULL, qkv, rows, 3 * hidden, hidden, 0, 1,
+                          1.0f, 0.0f, 0, 0);
+    if (r) round_through_half(qkv, rows * 3 * hidden);
+    hom_oracle_attention_f32in(qkv, cu, attn, bs, seq, heads, d, scale);
+    if (r) round_through_half(attn, rows * hidden);
+    hom_oracle_gemm_f32in(attn, wo, h, h, rows, hidden, hidden, hidden, rows,
+                          1.0f, 1.0f, 0, 0);
+    if (r) round_through_half(h, rows * hidden);
+    hom_oracle_layernorm_f32in(h, NULL, NULL, NULL, h, rows, hidden, eps);
+    if (r) round_through_half(h, rows * hidden);
+    hom_oracle_gemm_f32in(h, w1, NULL, f, rows, ffn, hidden, 0, 1, 1.0f, 0.0f,
+                          gelu_act, 0);
+    if (r) round_through_half(f, rows * ffn);
+    hom_oracle_gemm_f32in(f, w2, h, h, rows, hidden, ffn, hidden, rows, 1.0f,
+                          1.0f, 0, 0);
+    if (r) round_through_half(h, rows * hidden);
+    hom_oracle_layernorm_f32in(h, NULL, NULL, NULL, h, rows, hidden, eps);
+    if (r && l != layers - 1) round_through_half(h, rows * hidden);
+    free(wqkv);
+    free(wo);
+    free(w1);
+    free(w2);
   }
-  free(tmp);
   free(qkv);
   free(attn);
   free(f);

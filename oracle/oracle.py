@@ -58,7 +58,7 @@ def lib():
         L.hom_oracle_elementwise_f32.argtypes = ew
         L.hom_oracle_gather.argtypes = [c_void_p, c_void_p, c_void_p, c_int64, c_int64]
         L.hom_oracle_bert_encoder.argtypes = [c_void_p, c_void_p, c_void_p] + [c_int64] * 6 + \
-            [c_float, c_int, c_void_p]
+            [c_float, c_int, c_int]
         _lib = L
     return _lib
 
@@ -187,16 +187,19 @@ def gelu(x, form="erf"):
     return np.array([fn(float(v)) for v in np.asarray(x, np.float64).ravel()]).reshape(np.shape(x))
 
 
-def bert_encoder(h, weights, cu, layers, bs, seq, hidden, heads, ffn, eps=1e-12, gelu_form="erf"):
-    """h [bs*seq, hidden] f16 (copied), weights: flat f16 array of all layers
-    (Wqkv, Wo, W1, W2 per layer, each [K, N] row-major).  Returns (fp16 output,
-    fp32 value of the last layer norm before rounding)."""
-    h = _f16(h).copy()
+def bert_encoder(h, weights, cu, layers, bs, seq, hidden, heads, ffn, eps=1e-12, gelu_form="erf",
+                 round_intermediates=True):
+    """h [bs*seq, hidden] f16, weights: flat f16 array of all layers (Wqkv, Wo, W1,
+    W2 per layer, each [K, N] row-major).  round_intermediates=True rounds every
+    tensor the GPU path stores as fp16 (fp16-boundary-faithful); False keeps
+    them unrounded (pure fp32 reference).  Returns the final layer norm as
+    float32 [bs, seq, hidden], before its own rounding to fp16."""
+    h32 = np.ascontiguousarray(_f16(h).astype(np.float32)).reshape(bs * seq, hidden).copy()
     weights = _f16(weights)
     per_layer = hidden * 3 * hidden + hidden * hidden + 2 * hidden * ffn
     assert weights.size == layers * per_layer
     cu = np.ascontiguousarray(cu, np.int32)
-    out32 = np.empty((bs * seq, hidden), np.float32)
-    lib().hom_oracle_bert_encoder(_ptr(h), _ptr(weights), _ptr(cu), layers, bs, seq, hidden,
-                                  heads, ffn, eps, 1 if gelu_form == "erf" else 2, _ptr(out32))
-    return h.reshape(bs, seq, hidden), out32.reshape(bs, seq, hidden)
+    lib().hom_oracle_bert_encoder(_ptr(h32), _ptr(weights), _ptr(cu), layers, bs, seq, hidden,
+                                  heads, ffn, eps, 1 if gelu_form == "erf" else 2,
+                                  int(bool(round_intermediates)))
+    return h32.reshape(bs, seq, hidden)

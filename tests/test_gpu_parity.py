@@ -151,6 +151,14 @@ def test_gelu_kernel(gpu, rt, oracle):
 
 
 # -------------------------------------------------------------------- GEMM --
+def knum(rt, tile, epi="linear"):
+    """1-based manifest number of the kernel whose name holds `_<tile>_` and ends in `_<epi>`."""
+    for idx, name, _, _ in rt.manifest():
+        if f"_{tile}_" in name and name.endswith("_" + epi):
+            return idx + 1
+    raise KeyError((tile, epi))
+
+
 def run_gemm(gpu, rt, A, B, C, D_init, num, splitk, alpha=1.0, beta=0.0, act=0, in_place=False):
     M = rt.MemRef.from_tensor
     ta, tb = dev(A), dev(B)
@@ -200,14 +208,16 @@ def test_gemm_residual_in_place_and_batch_folding(gpu, rt, oracle):
     B = (g.standard_normal((1, K_, N_)) * 0.02).astype(np.float16)
     X = g.standard_normal((b, Mp, N_)).astype(np.float16)
     want = oracle.gemm(A.reshape(-1, K_), B[0], X.reshape(-1, N_), beta=1.0)
-    for num in (1, 4, 7):
+    for num in (knum(rt, "128x128_64x4"), knum(rt, "64x64_64x4"), knum(rt, "128x64_64x4"),
+                knum(rt, "128x128_32x2")):
         for sk in (1, 2, 6):
             got = run_gemm(gpu, rt, A, B, None, X, num, sk, beta=1.0, in_place=True)
             assert_close(got.reshape(-1, N_), want, **GEMM_TOL, what=f"in-place kernel {num} splitK {sk}")
     # [1, M', N] source shared by every batch, alpha/beta other than 1
     C1 = g.standard_normal((1, Mp, N_)).astype(np.float16)
     want = oracle.gemm(A.reshape(-1, K_), B[0], C1[0], alpha=0.5, beta=-2.0)
-    got = run_gemm(gpu, rt, A, B, C1, np.zeros((b, Mp, N_), np.float16), 1, 1, alpha=0.5, beta=-2.0)
+    got = run_gemm(gpu, rt, A, B, C1, np.zeros((b, Mp, N_), np.float16), knum(rt, "128x128_64x4"), 1,
+                   alpha=0.5, beta=-2.0)
     assert_close(got.reshape(-1, N_), want, **GEMM_TOL)
 
 
@@ -215,9 +225,10 @@ def test_gemm_split_k_is_deterministic_and_invariant(gpu, rt, oracle, synth):
     c = synth.skinny_gemm()  # M=64, K=4096, N=1024
     want = oracle.gemm(c["A"][0], c["B"][0])
     outs = {}
+    num = knum(rt, "64x64_64x4")
     for sk in (1, 2, 5, 8, 16):
-        a = run_gemm(gpu, rt, c["A"], c["B"], None, np.zeros((1, 64, 1024), np.float16), 4, sk)
-        b = run_gemm(gpu, rt, c["A"], c["B"], None, np.zeros((1, 64, 1024), np.float16), 4, sk)
+        a = run_gemm(gpu, rt, c["A"], c["B"], None, np.zeros((1, 64, 1024), np.float16), num, sk)
+        b = run_gemm(gpu, rt, c["A"], c["B"], None, np.zeros((1, 64, 1024), np.float16), num, sk)
         assert np.array_equal(a, b), f"split-K {sk} not reproducible"
         assert_close(a[0], want, **GEMM_TOL, what=f"skinny splitK={sk}")
         outs[sk] = a
@@ -229,13 +240,15 @@ def test_gemm_exact_cases(gpu, rt, literals):
     g = np.random.default_rng(33)
     A = g.standard_normal((1, 128, 128)).astype(np.float16)
     eye = np.eye(128, dtype=np.float16)[None]
-    for num in (1, 4, 25):
+    for num in (knum(rt, "128x128_64x4"), knum(rt, "64x64_64x8"), knum(rt, "64x64_64x2"),
+                knum(rt, "64x64_32x2_w2x2_nn_align1")):
         assert np.array_equal(run_gemm(gpu, rt, A, eye, None, np.zeros_like(A), num, 1), A)
         assert np.array_equal(run_gemm(gpu, rt, eye, A, None, np.zeros_like(A), num, 1), A)
     c = literals["gemm_const"]  # reference driver b.cu: 0.1 x 0.2 over K = 768
     A = np.full((1, c["m"], c["k"]), c["a"], np.float16)
     B = np.full((1, c["k"], c["n"]), c["b"], np.float16)
-    out = run_gemm(gpu, rt, A, B, None, np.zeros((1, c["m"], c["n"]), np.float16), 1, 1)
+    out = run_gemm(gpu, rt, A, B, None, np.zeros((1, c["m"], c["n"]), np.float16),
+                   knum(rt, "128x128_64x4"), 1)
     assert np.abs(out.astype(np.float64) - c["expect"]).max() < c["tol"]
 
 

@@ -284,9 +284,14 @@ def test_encoder_composition_matches_torch(oracle, gelu):
     h = _rand16(g, (bs * seq, hidden))
     lens = np.array([16, 5], np.int32)
     cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
-    out16, out32 = oracle.bert_encoder(h, weights, cu, layers, bs, seq, hidden, heads, ffn, gelu_form=gelu)
     want = _torch_encoder(h, weights, lens, layers, bs, seq, hidden, heads, ffn, gelu)
-    # fp16 rounding at every stored tensor: a few 1e-3 after two layers
+    # unrounded intermediates: agrees with the torch fp64 graph to fp32 precision
+    pure = oracle.bert_encoder(h, weights, cu, layers, bs, seq, hidden, heads, ffn, gelu_form=gelu,
+                               round_intermediates=False)
     for b in range(bs):
-        assert np.abs(out32[b, :lens[b]] - want[b, :lens[b]]).max() < 2e-2
-    assert np.array_equal(out16, out32.astype(np.float16))
+        assert np.abs(pure[b, :lens[b]] - want[b, :lens[b]]).max() < 2e-5
+    # fp16 rounding at every stored tensor: a few 1e-3 after two layers
+    out32 = oracle.bert_encoder(h, weights, cu, layers, bs, seq, hidden, heads, ffn, gelu_form=gelu)
+    for b in range(bs):
+        err = np.abs(out32[b, :lens[b]] - want[b, :lens[b]]).max()
+        assert 1e-5 < err < 2e-2
