@@ -9,18 +9,22 @@
 // Replaces the cuDNN fused attention reached through
 // include/NVGPUKernels/BertAttentionRunner.h:113-136.
 //
-// One wavefront owns 32 query rows; a workgroup of NW wavefronts shares the
-// K / V blocks (64 keys at a time) through LDS.  Both contractions run on
-// v_mfma_f32_32x32x16_f16 and are issued transposed:
-//   S^T = K Q^T   (A operand = K rows, B operand = Q rows, both contiguous in d)
+// A workgroup of NW wavefronts handles 32*NW query rows of one (batch, head);
+// each wavefront owns 32 of them.  Keys are walked in chunks of 128: the whole
+// workgroup stages the chunk's K and V rows into LDS (one barrier), then every
+// wavefront runs over it in blocks of 64 keys without further synchronisation.
+// Both contractions run on v_mfma_f32_32x32x16_f16 and are issued transposed:
+//   S^T = K Q^T   (A operand = K rows from LDS, B operand = Q rows in registers)
 //   O^T = V^T P^T (A operand = V columns, B operand = P rows)
 // With that orientation a lane holds, for ONE query row, 16 of the 32 scores of
 // a key sub-block, so the online-softmax row reductions are in-lane plus one
-// exchange with lane^32, and the probabilities are already laid out as the B
-// operand of the second MFMA: P never leaves registers.  The MFMA k index is
-// free as long as both operands agree, so V is read in the key order the score
-// accumulators happen to have.  V is staged as (key, key+1) half2 pairs so that
-// those reads are conflict-free 32-bit LDS loads.
+// exchange with lane^32, and the probabilities already have the layout of the
+// second MFMA's B operand: P never leaves registers.  The MFMA k index is free
+// as long as both operands agree, so V is read in the key order the score
+// accumulators happen to have: two runs of 4 consecutive keys per lane, each one
+// ds_read_b64_tr_b16 (the transposing LDS read) from the row-major V tile.
+// LDS rows are 128 bytes, unpadded; 16-byte chunks (K) / 64-byte groups (V) are
+// XOR-permuted by row so that the fragment reads are bank-conflict free.
 #include "kernels.h"
 
 namespace hom {
@@ -29,21 +33,30 @@ namespace {
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef _Float16 half4 __attribute__((ext_vector_type(4)));
 typedef float float16v __attribute__((ext_vector_type(16)));
-typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
+typedef short short4v __attribute__((ext_vector_type(4)));
+typedef short short8v __attribute__((ext_vector_type(8)));
 
 constexpr int kWave = 64;
 constexpr int kHeadDim = 64;
-constexpr int kKeyBlock = 64;
-constexpr int K_LD = kHeadDim + 8;  // halves per LDS row of K
-constexpr int VP_LD = kHeadDim + 16; // dwords per LDS row of key-pair-packed V
+constexpr int kChunk = 128;                  // keys staged per barrier
+constexpr int kTileBytes = kChunk * 128;     // one K or V chunk in LDS
+
+// chunk c (16 bytes) of K row r lives at position c ^ ((r >> 1) & 7)
+__device__ __forceinline__ int swzK(int row, int chunk) {
+  return chunk ^ ((row >> 1) & 7);
+}
+// 64-byte group g of V row k lives at position g ^ ((k >> 1) & 1)
+__device__ __forceinline__ int swzV(int k, int group) {
+  return group ^ ((k >> 1) & 1);
+}
 
 template <int NW>
 __global__ __launch_bounds__(NW *kWave) void bertAttentionKernel(
     const _Float16 *__restrict__ qkv, const int32_t *__restrict__ cu,
     _Float16 *__restrict__ out, int seq, int heads, float scale) {
   constexpr int kThreads = NW * kWave;
-  __shared__ __attribute__((aligned(16))) _Float16 sK[kKeyBlock * K_LD];
-  __shared__ __attribute__((aligned(16))) uint32_t sV[(kKeyBlock / 2) * VP_LD];
+  __shared__ __attribute__((aligned(16))) unsigned char sK[kTileBytes];
+  __shared__ __attribute__((aligned(16))) unsigned char sV[kTileBytes];
 
   const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
   const int l32 = lane % 32, hb = lane / 32;
@@ -77,7 +90,8 @@ __global__ __launch_bounds__(NW *kWave) void bertAttentionKernel(
   }
 
   // Q fragments (B operand of S^T = K Q^T): lane (q = l32, hb) holds
-  // Q[q][kk*16 + hb*8 .. +8] for kk = 0..3.
+  // Q[q][kk*16 + hb*8 .. +8] for kk = 0..3, pre-multiplied by nothing: the scale
+  // is applied to the fp32 scores.
   half8 fq[kHeadDim / 16];
   {
     const int q = q0 + l32;
@@ -102,126 +116,120 @@ __global__ __launch_bounds__(NW *kWave) void bertAttentionKernel(
       accO[d][e] = 0.f;
   float rowMax = -INFINITY, rowSum = 0.f;
 
-  // The whole workgroup walks the same key blocks (uniform trip count).
-  const int numBlocks = (len + kKeyBlock - 1) / kKeyBlock;
-  for (int kbIdx = 0; kbIdx < numBlocks; kbIdx++) {
-    const int key0 = kbIdx * kKeyBlock;
-    __syncthreads(); // previous block fully consumed
-    // ---- stage K: 64 keys x 8 vectors of 16 bytes ----
-    for (int v = tid; v < kKeyBlock * (kHeadDim / 8); v += kThreads) {
-      const int r = v / (kHeadDim / 8), c = (v % (kHeadDim / 8)) * 8;
-      half8 val;
+  // Per-lane constants of the fragment addresses.
+  const int swzLane = (l32 >> 1) & 7;          // K: (row >> 1) & 7 for row = 32*x + l32
+  const int trRow = (lane % 16) / 4;           // V: source row inside a run of 4 keys
+  const int trCol = ((lane % 32) / 16) * 16 + (lane % 4) * 4;
+  const int vSwz = (trRow >> 1) & 1;           // key bases are multiples of 4
+
+  const int numChunks = (len + kChunk - 1) / kChunk; // uniform over the workgroup
+  for (int ch = 0; ch < numChunks; ch++) {
+    const int key0 = ch * kChunk;
+    // keys of this chunk that any wavefront will touch, rounded up to a block
+    const int live = (len - key0 < kChunk ? ((len - key0 + 63) / 64) * 64 : kChunk);
+    if (ch > 0)
+      __syncthreads(); // previous chunk fully consumed
+    // ---- stage K and V rows [key0, key0 + live): 8 vectors of 16 bytes per row.
+    // Rows past the sequence end are zero-filled: masked scores ignore K, but a
+    // masked probability (0) times a non-finite V would poison the output.
+    for (int v = tid; v < live * 8; v += kThreads) {
+      const int r = v / 8, c = v % 8;
+      half8 kv, vv;
 #pragma unroll
       for (int e = 0; e < 8; e++)
-        val[e] = _Float16(0);
-      if (key0 + r < seq)
-        val = *reinterpret_cast<const half8 *>(
-            kBase + int64_t(key0 + r) * tokStride + c);
-      *reinterpret_cast<half8 *>(sK + r * K_LD + c) = val;
-    }
-    // ---- stage V as (key, key+1) pairs ----
-    for (int v = tid; v < (kKeyBlock / 2) * (kHeadDim / 8); v += kThreads) {
-      const int kp = v / (kHeadDim / 8), c = (v % (kHeadDim / 8)) * 8;
-      half8 v0, v1;
-#pragma unroll
-      for (int e = 0; e < 8; e++)
-        v0[e] = v1[e] = _Float16(0);
-      const int key = key0 + 2 * kp;
-      if (key < seq)
-        v0 = *reinterpret_cast<const half8 *>(vBase + int64_t(key) * tokStride +
-                                              c);
-      if (key + 1 < seq)
-        v1 = *reinterpret_cast<const half8 *>(
-            vBase + int64_t(key + 1) * tokStride + c);
-      half8 lo, hi;
-#pragma unroll
-      for (int e = 0; e < 4; e++) {
-        lo[2 * e] = v0[e];
-        lo[2 * e + 1] = v1[e];
-        hi[2 * e] = v0[4 + e];
-        hi[2 * e + 1] = v1[4 + e];
+        kv[e] = vv[e] = _Float16(0);
+      if (key0 + r < len) {
+        kv = *reinterpret_cast<const half8 *>(kBase + int64_t(key0 + r) * tokStride + c * 8);
+        vv = *reinterpret_cast<const half8 *>(vBase + int64_t(key0 + r) * tokStride + c * 8);
       }
-      *reinterpret_cast<half8 *>(sV + kp * VP_LD + c) = lo;
-      *reinterpret_cast<half8 *>(sV + kp * VP_LD + c + 4) = hi;
+      *reinterpret_cast<half8 *>(sK + r * 128 + swzK(r, c) * 16) = kv;
+      *reinterpret_cast<half8 *>(sV + r * 128 + swzV(r, c / 4) * 64 + (c % 4) * 16) = vv;
     }
     __syncthreads();
 
-    // ---- S^T = K Q^T for two 32-key sub-blocks ----
-    float16v accS[2];
+    for (int blk = 0; blk < live; blk += 64) {
+      // ---- S^T = K Q^T for two 32-key sub-blocks ----
+      float16v accS[2];
 #pragma unroll
-    for (int sb = 0; sb < 2; sb++) {
+      for (int sb = 0; sb < 2; sb++) {
 #pragma unroll
-      for (int e = 0; e < 16; e++)
-        accS[sb][e] = 0.f;
+        for (int e = 0; e < 16; e++)
+          accS[sb][e] = 0.f;
 #pragma unroll
-      for (int kk = 0; kk < kHeadDim / 16; kk++) {
-        const half8 fk = *reinterpret_cast<const half8 *>(
-            sK + (sb * 32 + l32) * K_LD + kk * 16 + hb * 8);
-        accS[sb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fk, fq[kk], accS[sb],
-                                                          0, 0, 0);
+        for (int kk = 0; kk < kHeadDim / 16; kk++) {
+          const half8 fk = *reinterpret_cast<const half8 *>(
+              sK + (blk + sb * 32 + l32) * 128 + ((kk * 2 + hb) ^ swzLane) * 16);
+          accS[sb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fk, fq[kk], accS[sb],
+                                                            0, 0, 0);
+        }
       }
-    }
-    // accS[sb][e] is the score of query l32 against key
-    //   key0 + sb*32 + 8*(e/4) + 4*hb + e%4.
-    float blockMax = -INFINITY;
+      // accS[sb][e] is the score of query l32 against key
+      //   key0 + blk + sb*32 + 8*(e/4) + 4*hb + e%4.
+      float blockMax = -INFINITY;
 #pragma unroll
-    for (int sb = 0; sb < 2; sb++)
+      for (int sb = 0; sb < 2; sb++)
 #pragma unroll
-      for (int e = 0; e < 16; e++) {
-        const int key = key0 + sb * 32 + 8 * (e / 4) + 4 * hb + (e % 4);
-        const float s = key < len ? accS[sb][e] * scale : -INFINITY;
-        accS[sb][e] = s;
-        blockMax = fmaxf(blockMax, s);
-      }
-    blockMax = fmaxf(blockMax, __shfl_xor(blockMax, 32, kWave));
-    const float newMax = fmaxf(rowMax, blockMax);
-    // Every block that is visited has at least one valid key, so newMax is
-    // finite and the differences below are never inf - inf.
-    const float corr = __expf(rowMax - newMax);
-    float blockSum = 0.f;
+        for (int e = 0; e < 16; e++) {
+          const int key = key0 + blk + sb * 32 + 8 * (e / 4) + 4 * hb + (e % 4);
+          const float s = key < len ? accS[sb][e] * scale : -INFINITY;
+          accS[sb][e] = s;
+          blockMax = fmaxf(blockMax, s);
+        }
+      blockMax = fmaxf(blockMax, __shfl_xor(blockMax, 32, kWave));
+      const float newMax = fmaxf(rowMax, blockMax);
+      // Every block that is visited has at least one valid key, so newMax is
+      // finite and the differences below are never inf - inf.
+      const float corr = __expf(rowMax - newMax);
+      float blockSum = 0.f;
 #pragma unroll
-    for (int sb = 0; sb < 2; sb++)
+      for (int sb = 0; sb < 2; sb++)
 #pragma unroll
-      for (int e = 0; e < 16; e++) {
-        const float pv = __expf(accS[sb][e] - newMax);
-        accS[sb][e] = pv;
-        blockSum += pv;
-      }
-    blockSum += __shfl_xor(blockSum, 32, kWave);
-    rowSum = rowSum * corr + blockSum;
-    rowMax = newMax;
+        for (int e = 0; e < 16; e++) {
+          const float pv = __expf(accS[sb][e] - newMax);
+          accS[sb][e] = pv;
+          blockSum += pv;
+        }
+      blockSum += __shfl_xor(blockSum, 32, kWave);
+      rowSum = rowSum * corr + blockSum;
+      rowMax = newMax;
 #pragma unroll
-    for (int d = 0; d < 2; d++)
+      for (int d = 0; d < 2; d++)
 #pragma unroll
-      for (int e = 0; e < 16; e++)
-        accO[d][e] *= corr;
+        for (int e = 0; e < 16; e++)
+          accO[d][e] *= corr;
 
-    // ---- O^T += V^T P^T ----
+      // ---- O^T += V^T P^T ----
 #pragma unroll
-    for (int sb = 0; sb < 2; sb++) {
+      for (int sb = 0; sb < 2; sb++) {
 #pragma unroll
-      for (int t = 0; t < 2; t++) {
-        // B operand: P[q][key(hb, e)], key(hb, e) = sb*32 + 8*(2t + e/4) + 4*hb
-        // + e%4, which is accumulators 8t .. 8t+7 of this lane.
-        half8 fp;
+        for (int t = 0; t < 2; t++) {
+          // B operand: P[q][key(hb, e)], key(hb, e) = sb*32 + 8*(2t + e/4) + 4*hb
+          // + e%4, which is accumulators 8t .. 8t+7 of this lane.
+          half8 fp;
 #pragma unroll
-        for (int e = 0; e < 8; e++)
-          fp[e] = _Float16(accS[sb][8 * t + e]);
+          for (int e = 0; e < 8; e++)
+            fp[e] = _Float16(accS[sb][8 * t + e]);
 #pragma unroll
-        for (int d = 0; d < 2; d++) {
-          // A operand: V[key(hb, e)][d*32 + l32]; keys come in two runs of 4 =
-          // two pairs each.
-          uint4v w;
+          for (int d = 0; d < 2; d++) {
+            // A operand: V[key(hb, e)][d*32 + l32]: two runs of 4 consecutive
+            // keys, each transposed out of 4 V rows x 16 columns by one read.
+            short4v run[2];
 #pragma unroll
-          for (int g = 0; g < 2; g++) {
-            const int keyLocal = sb * 32 + 8 * (2 * t + g) + 4 * hb;
-            const int kp = keyLocal / 2;
-            w[2 * g] = sV[kp * VP_LD + d * 32 + l32];
-            w[2 * g + 1] = sV[(kp + 1) * VP_LD + d * 32 + l32];
+            for (int g = 0; g < 2; g++) {
+              const int keyLocal = blk + sb * 32 + 8 * (2 * t + g) + 4 * hb + trRow;
+              run[g] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                  (__attribute__((address_space(3))) short4v *)(
+                      sV + keyLocal * 128 + (d ^ vSwz) * 64 + trCol * 2));
+            }
+            short8v both;
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+              both[e] = run[0][e];
+              both[4 + e] = run[1][e];
+            }
+            accO[d] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+                __builtin_bit_cast(half8, both), fp, accO[d], 0, 0, 0);
           }
-          const half8 fv = __builtin_bit_cast(half8, w);
-          accO[d] =
-              __builtin_amdgcn_mfma_f32_32x32x16_f16(fv, fp, accO[d], 0, 0, 0);
         }
       }
     }
@@ -263,25 +271,23 @@ Status launchBertAttentionF16(const _Float16 *qkv, const int32_t *cuSeqlens,
                 Status::kInvalidArgument, "attention: misaligned operands");
   if (bs == 0 || seq == 0 || heads == 0)
     return Status::kSuccess;
-  // Fewer wavefronts per workgroup when there are few (batch, head) pairs, so
-  // that short sequences still spread over the chip.
+  // 128 query rows per workgroup when that still gives every CU work,
+  // otherwise 64 (K/V of a (batch, head) are then staged by two workgroups).
   const int cus = deviceInfo().computeUnits;
   const int64_t pairs = bs * heads;
-  if (pairs * ((seq + 127) / 128) >= 2 * int64_t(cus)) {
+  bool wide = pairs * ((seq + 127) / 128) >= int64_t(cus) || seq <= 32;
+  if (const char *force = getenv("HOM_ATTENTION_WAVES")) // profiling knob: 2 or 4
+    wide = atoi(force) == 4;
+  if (wide) {
     dim3 grid((unsigned)((seq + 127) / 128), (unsigned)heads, (unsigned)bs);
     bertAttentionKernel<4><<<grid, dim3(256), 0, s>>>(qkv, cuSeqlens, out,
                                                       int(seq), int(heads),
                                                       scale);
-  } else if (pairs * ((seq + 63) / 64) >= int64_t(cus)) {
+  } else {
     dim3 grid((unsigned)((seq + 63) / 64), (unsigned)heads, (unsigned)bs);
     bertAttentionKernel<2><<<grid, dim3(128), 0, s>>>(qkv, cuSeqlens, out,
                                                       int(seq), int(heads),
                                                       scale);
-  } else {
-    dim3 grid((unsigned)((seq + 31) / 32), (unsigned)heads, (unsigned)bs);
-    bertAttentionKernel<1><<<grid, dim3(64), 0, s>>>(qkv, cuSeqlens, out,
-                                                     int(seq), int(heads),
-                                                     scale);
   }
   HOM_HIP_RET(hipGetLastError(), Status::kInternal);
   return Status::kSuccess;

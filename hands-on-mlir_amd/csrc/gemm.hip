@@ -43,6 +43,8 @@
 //    B is interleaved into (k, k+1) half2 pairs while it is staged.
 #include "kernels.h"
 
+#include <type_traits>
+
 namespace hom {
 namespace {
 
@@ -486,6 +488,265 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmDmaKernel(GemmParams p) {
 #endif
 }
 
+// ==================================================================== pipe ==
+// Same LDS layout, fragment reads and barrier placement as the dma kernels, but
+// the slabs travel global -> registers -> LDS (two LDS buffers): the loads of
+// slab i+1 are issued before slab i is multiplied and written to LDS after it.
+// The vector memory path into registers sustains several times the bandwidth
+// of the LDS-DMA path on this chip, which matters once a CU streams more than
+// ~16 bytes per clock (large tiles, or several workgroups per CU).
+template <int BM, int BN, int WM, int WN, int DIST, int EPI, bool B_NK>
+__global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(GemmParams p) {
+  constexpr int BK = 64;
+  constexpr int THREADS = WM * WN * kWave;
+  constexpr int WTM = BM / WM, WTN = BN / WN;
+  constexpr int MI = WTM / 32, NI = WTN / 32;
+  constexpr int A_BYTES = BM * BK * 2, B_BYTES = BN * BK * 2;
+  constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
+  constexpr int A_VECS = A_BYTES / 16, B_VECS = B_BYTES / 16;
+  static_assert(A_VECS % THREADS == 0 && B_VECS % THREADS == 0,
+                "tile must split evenly over the threads");
+  constexpr int A_PER_T = A_VECS / THREADS, B_PER_T = B_VECS / THREADS;
+  constexpr int B_ROW_BYTES = B_NK ? 128 : BN * 2;
+  constexpr int B_VPR = B_ROW_BYTES / 16; // vectors per LDS row of B
+  constexpr int KSTEPS = BK / 16;
+
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+
+  const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+  const int waveM = wave / WN, waveN = wave % WN;
+  const int l32 = lane % 32, kb = lane / 32;
+
+  const int nTiles = p.tilesM * p.tilesN;
+  const int tile = tileForBlock(nTiles);
+  int tileM, tileN;
+  tileCoords(tile, p.tilesM, p.tilesN, &tileM, &tileN);
+  const int m0 = tileM * BM, n0 = tileN * BN;
+  const int slice = blockIdx.y, numSlices = gridDim.y;
+  const int kTiles = (p.K + BK - 1) / BK;
+  const int ktBegin = slice * p.kTilesPerSlice;
+  int ktEnd = ktBegin + p.kTilesPerSlice;
+  if (ktEnd > kTiles)
+    ktEnd = kTiles;
+
+  // ---- global sources: a uniform tile base plus a constant 32-bit element
+  // offset per thread.  Rows / columns past the edge are clamped to the last
+  // valid one: what they fetch only reaches outputs that are never stored, so
+  // full slabs need no predication (the K tail does).
+  const _Float16 *aTile = p.A + int64_t(m0) * p.lda;
+  const _Float16 *bTile = B_NK ? p.B + int64_t(n0) * p.ldb : p.B + n0;
+  uint32_t aOff[A_PER_T], bOff[B_PER_T];
+  int aDst[A_PER_T], bDst[B_PER_T];
+  int aK[A_PER_T], bK[B_PER_T]; // k position inside the slab (for the tail)
+#pragma unroll
+  for (int i = 0; i < A_PER_T; i++) {
+    const int v = tid + i * THREADS;
+    const int r = v / 8, c = v % 8;
+    const int rr = m0 + r < p.M ? r : p.M - 1 - m0;
+    aK[i] = c * 8;
+    aOff[i] = uint32_t(rr) * uint32_t(p.lda) + c * 8;
+    aDst[i] = r * 128 + swzK(r, c) * 16;
+  }
+#pragma unroll
+  for (int i = 0; i < B_PER_T; i++) {
+    const int v = tid + i * THREADS;
+    const int r = v / B_VPR, c = v % B_VPR;
+    if (B_NK) {
+      const int rr = n0 + r < p.N ? r : p.N - 1 - n0;
+      bK[i] = c * 8;
+      bOff[i] = uint32_t(rr) * uint32_t(p.ldb) + c * 8;
+      bDst[i] = r * 128 + swzK(r, c) * 16;
+    } else {
+      const int cc = n0 + c * 8 < p.N ? c * 8 : p.N - 8 - n0;
+      bK[i] = r;
+      bOff[i] = uint32_t(r) * uint32_t(p.ldb) + cc;
+      bDst[i] = r * B_ROW_BYTES + swzN<BN>(r, c / 4) * 64 + (c % 4) * 16;
+    }
+  }
+
+  half8 regA[DIST][A_PER_T], regB[DIST][B_PER_T];
+  auto zero8 = []() {
+    half8 z;
+#pragma unroll
+    for (int e = 0; e < 8; e++)
+      z[e] = _Float16(0);
+    return z;
+  };
+  auto loadGlobal = [&](int kt, auto setC) {
+    constexpr int S = decltype(setC)::value;
+    const int k0 = kt * BK;
+    const _Float16 *aSlab = aTile + k0;
+    const _Float16 *bSlab = B_NK ? bTile + k0 : bTile + int64_t(k0) * p.ldb;
+    if (k0 + BK <= p.K) {
+#pragma unroll
+      for (int i = 0; i < A_PER_T; i++)
+        regA[S][i] = *reinterpret_cast<const half8 *>(aSlab + aOff[i]);
+#pragma unroll
+      for (int i = 0; i < B_PER_T; i++)
+        regB[S][i] = *reinterpret_cast<const half8 *>(bSlab + bOff[i]);
+    } else {
+#pragma unroll
+      for (int i = 0; i < A_PER_T; i++)
+        regA[S][i] = k0 + aK[i] < p.K
+                      ? *reinterpret_cast<const half8 *>(aSlab + aOff[i])
+                      : zero8();
+#pragma unroll
+      for (int i = 0; i < B_PER_T; i++)
+        regB[S][i] = k0 + bK[i] < p.K
+                      ? *reinterpret_cast<const half8 *>(bSlab + bOff[i])
+                      : zero8();
+    }
+  };
+  auto storeLds = [&](int stage, auto setC) {
+    constexpr int S = decltype(setC)::value;
+    unsigned char *sA = smem + stage * STAGE_BYTES;
+    unsigned char *sB = sA + A_BYTES;
+#pragma unroll
+    for (int i = 0; i < A_PER_T; i++)
+      *reinterpret_cast<half8 *>(sA + aDst[i]) = regA[S][i];
+#pragma unroll
+    for (int i = 0; i < B_PER_T; i++)
+      *reinterpret_cast<half8 *>(sB + bDst[i]) = regB[S][i];
+  };
+
+  float16v acc[MI][NI];
+#pragma unroll
+  for (int i = 0; i < MI; i++)
+#pragma unroll
+    for (int j = 0; j < NI; j++)
+#pragma unroll
+      for (int e = 0; e < 16; e++)
+        acc[i][j][e] = 0.f;
+
+  // ---- fragment addresses: a few per-lane bases, the rest are immediates ----
+  // K-contiguous tiles: the swizzle term (row >> 1) & 7 only involves bits of
+  // lane % 32 (wave / block offsets are multiples of 32), so the chunk position
+  // of k step kk is the same for every 32-row block of the wavefront.
+  const int swzLane = (l32 >> 1) & 7;
+  int aFrag[KSTEPS], bFragK[KSTEPS];
+#pragma unroll
+  for (int kk = 0; kk < KSTEPS; kk++) {
+    aFrag[kk] = (waveM * WTM + l32) * 128 + ((kk * 2 + kb) ^ swzLane) * 16;
+    bFragK[kk] =
+        A_BYTES + (waveN * WTN + l32) * 128 + ((kk * 2 + kb) ^ swzLane) * 16;
+  }
+  // Row-major B, transposing reads: source lane L = lane % 16 of a 16-lane group
+  // supplies row kbase + L/4 and the 4 columns at (L%4)*4 of the group's 16
+  // columns.  k & 3 == L/4 for every (kk, kb, h), so the 64-byte group swizzle
+  // is a per-lane constant as well.
+  const int trRow = (lane % 16) / 4;
+  const int trCol = ((lane % 32) / 16) * 16 + (lane % 4) * 4;
+  int bFragN[NI];
+#pragma unroll
+  for (int j = 0; j < NI; j++) {
+    const int group = (waveN * WTN) / 32 + j;
+    bFragN[j] = A_BYTES + (kb * 8 + trRow) * B_ROW_BYTES +
+                swzN<BN>(trRow, group) * 64 + trCol * 2;
+  }
+
+  auto loadFrags = [&](int stage, int kk, half8 (&fa)[MI], half8 (&fb)[NI]) {
+    const unsigned char *st = smem + stage * STAGE_BYTES;
+#pragma unroll
+    for (int i = 0; i < MI; i++)
+      fa[i] = *reinterpret_cast<const half8 *>(st + aFrag[kk] + i * 32 * 128);
+    if (B_NK) {
+#pragma unroll
+      for (int j = 0; j < NI; j++)
+        fb[j] = *reinterpret_cast<const half8 *>(st + bFragK[kk] + j * 32 * 128);
+    } else {
+#pragma unroll
+      for (int j = 0; j < NI; j++) {
+        short4v t[2];
+#pragma unroll
+        for (int h = 0; h < 2; h++)
+          t[h] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+              (__attribute__((address_space(3))) short4v *)(
+                  st + bFragN[j] + (kk * 16 + h * 4) * B_ROW_BYTES));
+        typedef short short8v __attribute__((ext_vector_type(8)));
+        short8v both;
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          both[e] = t[0][e];
+          both[4 + e] = t[1][e];
+        }
+        fb[j] = __builtin_bit_cast(half8, both);
+      }
+    }
+  };
+  auto mfmaStep = [&](half8 (&fa)[MI], half8 (&fb)[NI]) {
+#pragma unroll
+    for (int i = 0; i < MI; i++)
+#pragma unroll
+      for (int j = 0; j < NI; j++)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[j], fa[i],
+                                                           acc[i][j], 0, 0, 0);
+  };
+
+  // ---- main loop ----
+  // LDS holds slab i (buffer i & 1); slab i+1 sits in registers (or is on its way
+  // there) and is written to the other buffer after the third k step; with
+  // DIST == 2 the register set that was just written out is refilled with slab
+  // i+3 at once, so two slabs of global loads are in flight per workgroup -- on
+  // this chip one slab per CU in flight is not enough to cover memory latency.
+  // The barrier is a bare s_barrier behind an LDS-only wait: a fence here would
+  // drain the global loads that were just issued.
+  using Set0 = std::integral_constant<int, 0>;
+  using Set1 = std::integral_constant<int, DIST - 1>;
+  half8 fa[2][MI], fb[2][NI];
+  const int nk = ktEnd - ktBegin;
+  auto slab = [&](int i, auto setC) {
+    const int cur = i & 1;
+    const bool more = i + 1 < nk;
+    if (DIST == 1 && more)
+      loadGlobal(ktBegin + i + 1, setC);
+#pragma unroll
+    for (int kk = 0; kk < KSTEPS - 1; kk++) {
+      loadFrags(cur, kk + 1, fa[(kk + 1) & 1], fb[(kk + 1) & 1]);
+      mfmaStep(fa[kk & 1], fb[kk & 1]);
+    }
+    if (more) {
+      // The other buffer was last read before the previous barrier, so it can
+      // be overwritten now; after this barrier every wavefront has its last
+      // fragments of slab i in registers and slab i+1 is visible.
+      storeLds(cur ^ 1, setC);
+      if (DIST == 2 && i + 3 < nk)
+        loadGlobal(ktBegin + i + 3, setC);
+      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+      loadFrags(cur ^ 1, 0, fa[0], fb[0]);
+    }
+    mfmaStep(fa[(KSTEPS - 1) & 1], fb[(KSTEPS - 1) & 1]);
+  };
+  if (nk > 0) {
+    loadGlobal(ktBegin, Set0{});
+    storeLds(0, Set0{});
+    if (DIST == 2) {
+      if (nk > 1)
+        loadGlobal(ktBegin + 1, Set1{});
+      if (nk > 2)
+        loadGlobal(ktBegin + 2, Set0{});
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    loadFrags(0, 0, fa[0], fb[0]);
+    if (DIST == 1) {
+      for (int i = 0; i < nk; i++)
+        slab(i, Set0{});
+    } else {
+      // slab i+1 lives in register set (i+1) & 1
+      for (int i = 0; i < nk; i += 2) {
+        slab(i, Set1{});
+        if (i + 1 < nk)
+          slab(i + 1, Set0{});
+      }
+    }
+  }
+
+  if (numSlices > 1) {
+    storePartial<MI, NI, THREADS>(p, acc, tile, slice, numSlices, tid);
+    return;
+  }
+  epilogueStore<MI, NI, WTM, WTN, EPI, 8>(p, acc, m0, n0, waveM, waveN, lane);
+}
+
 // ================================================================== staged ==
 // VEC == 8: N, K multiples of 8 and 16-byte aligned operands (128-bit global
 // accesses).  VEC == 1: any shape/alignment, scalar global accesses.
@@ -874,6 +1135,28 @@ Status launchDma(const GemmProblem &pr, hipStream_t s) {
   return Status::kSuccess;
 }
 
+template <int BM, int BN, int WM, int WN, int DIST, int EPI, bool B_NK>
+Status launchPipe(const GemmProblem &pr, hipStream_t s) {
+  constexpr int SMEM = 2 * (BM + BN) * 64 * 2;
+  LaunchPlan plan;
+  Status st = planLaunch<BM, BN, 64>(pr, &plan);
+  if (st != Status::kSuccess)
+    return st;
+  auto kernel = gemmPipeKernel<BM, BN, WM, WN, DIST, EPI, B_NK>;
+  static bool attrSet = false;
+  st = allowLds(kernel, SMEM, &attrSet);
+  if (st != Status::kSuccess)
+    return st;
+  if (plan.nTiles == 0)
+    return Status::kSuccess;
+  kernel<<<dim3((unsigned)plan.nTiles, (unsigned)plan.splitK),
+           dim3(WM * WN * kWave), SMEM, s>>>(plan.p);
+  HOM_HIP_RET(hipGetLastError(), Status::kInternal);
+  if (plan.splitK > 1)
+    return launchReduce<BM, BN, WM, WN, EPI, 8>(plan, s);
+  return Status::kSuccess;
+}
+
 using LaunchFn = Status (*)(const GemmProblem &, hipStream_t);
 
 struct KernelEntry {
@@ -898,6 +1181,21 @@ struct KernelEntry {
   HOM_DMA_ENTRY(BM, BN, WM, WN, NS, Epilogue::kLinear, "linear", 0),           \
       HOM_DMA_ENTRY(BM, BN, WM, WN, NS, Epilogue::kGeluErf, "gelu", 1),        \
       HOM_DMA_ENTRY(BM, BN, WM, WN, NS, Epilogue::kGeluTanh, "gelutanh", 1)
+
+// "r<d>" after the LDS stage count marks the register-staged pipeline with d
+// slabs of global loads in flight.
+#define HOM_PIPE_ENTRY(BM, BN, WM, WN, DIST, EPI_ENUM, EPI_STR, ACT)           \
+  {                                                                            \
+    {"hom_gfx950_mfma_f16_s32x32x16gemm_f16_" #BM "x" #BN "_64x2r" #DIST       \
+     "_w" #WM "x" #WN "_nn_align8_" EPI_STR,                                   \
+     BM, BN, 64, WM, WN, 8, ACT, EPI_ENUM},                                    \
+        launchPipe<BM, BN, WM, WN, DIST, int(EPI_ENUM), false>,                \
+        launchPipe<BM, BN, WM, WN, DIST, int(EPI_ENUM), true>                  \
+  }
+#define HOM_PIPE_TILE(BM, BN, WM, WN, DIST)                                    \
+  HOM_PIPE_ENTRY(BM, BN, WM, WN, DIST, Epilogue::kLinear, "linear", 0),        \
+      HOM_PIPE_ENTRY(BM, BN, WM, WN, DIST, Epilogue::kGeluErf, "gelu", 1),     \
+      HOM_PIPE_ENTRY(BM, BN, WM, WN, DIST, Epilogue::kGeluTanh, "gelutanh", 1)
 
 #define HOM_STAGED_ENTRY(BM, BN, BK, WM, WN, EPI_ENUM, EPI_STR, ACT, VEC)      \
   {                                                                            \
@@ -930,6 +1228,18 @@ const KernelEntry kKernels[] = {
     HOM_DMA_TILE(256, 128, 4, 2, 3),
     HOM_DMA_TILE(256, 256, 2, 4, 2),
     HOM_DMA_TILE(128, 256, 2, 4, 3),
+    HOM_PIPE_TILE(64, 64, 2, 2, 1),
+    HOM_PIPE_TILE(128, 64, 2, 2, 1),
+    HOM_PIPE_TILE(64, 128, 2, 2, 1),
+    HOM_PIPE_TILE(128, 128, 2, 2, 1),
+    HOM_PIPE_TILE(128, 128, 2, 4, 1),
+    HOM_PIPE_TILE(256, 256, 2, 4, 1),
+    HOM_PIPE_TILE(64, 64, 2, 2, 2),
+    HOM_PIPE_TILE(128, 128, 2, 2, 2),
+    HOM_PIPE_TILE(128, 128, 2, 4, 2),
+    HOM_PIPE_TILE(256, 128, 4, 2, 2),
+    HOM_PIPE_TILE(128, 256, 2, 4, 2),
+    HOM_PIPE_TILE(256, 256, 2, 4, 2),
     HOM_STAGED_TILE(128, 128, 32, 2, 2, 8),
     HOM_STAGED_TILE(64, 64, 64, 2, 2, 8),
     HOM_STAGED_TILE(64, 64, 32, 2, 2, 1),
