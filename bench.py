@@ -81,7 +81,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this path runs on one GPU; --gpus N with N > 1 is not supported "
-                 "(the workload shards by batch with no exchange step, see DESIGN.md)")
+                 "(the workload shards by batch with no exchange step between GPUs)")
 
     import numpy as np
     import torch
@@ -117,10 +117,14 @@ def main():
     g_ms = drv.homTimeGemm(M, N, K, 2, 1, idx.value + 1, sk.value, 2000, 50)
     g_flops = 2.0 * M * N * K
     achieved = g_flops / (g_ms * 1e-3) / 1e12
+    # HBM bytes per launch of this kernel from the rocprofv3 FETCH_SIZE / WRITE_SIZE runs
+    # (measured offline, scaled by a plain copy; summary beside the figure)
     traffic = None
-    tpath = os.path.join(ROOT, "profiles", "traffic.json")
+    tpath = os.path.join(ROOT, "profiles", "traffic.txt")
     if os.path.exists(tpath):
-        traffic = json.load(open(tpath)).get("gemm_bias_gelu_1024x3072x768")
+        for line in open(tpath):
+            if line.startswith("gemm1 "):
+                traffic = float(line.split()[1])
 
     def gbs(nbytes, t_ms):
         return nbytes / (t_ms * 1e-3) / 1e9

@@ -384,8 +384,20 @@ bool GemmProfiler::ensure(Buffer &b, int64_t elems) {
                 (long long)elems);
     return false;
   }
-  // Zeros: timing does not depend on the values, and NaN patterns are avoided.
-  (void)hipMemset(p, 0, size_t(elems) * sizeof(_Float16));
+  // Random finite values: on this GPU the clock under MFMA load depends on how
+  // much the operands toggle, so all-zero buffers would flatter every kernel.
+  {
+    std::vector<_Float16> host(static_cast<size_t>(elems));
+    uint32_t x = 0x9E3779B9u ^ uint32_t(elems);
+    for (auto &v : host) {
+      x ^= x << 13;
+      x ^= x >> 17;
+      x ^= x << 5;
+      v = _Float16((float(x & 0xffff) / 32768.0f - 1.0f) * 0.5f);
+    }
+    (void)hipMemcpy(p, host.data(), size_t(elems) * sizeof(_Float16),
+                    hipMemcpyHostToDevice);
+  }
   b.data = static_cast<_Float16 *>(p);
   b.capacity = elems;
   return true;

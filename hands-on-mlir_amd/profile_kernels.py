@@ -1,0 +1,54 @@
+"""Tiny single-kernel workloads to run under rocprofv3 (kernel trace or --pmc).
+
+    python3 hands-on-mlir_amd/profile_kernels.py <what> [iters]
+
+what:  gemm1      FFN1 GEMM + bias + tanh-GELU, M=1024 K=768 N=3072 (tuned kernel)
+       gemm5      BERT-large FFN2 GEMM, M=16384 K=4096 N=1024
+       layernorm  in-place layer norm, 16384 x 1024
+       attention  packed-QKV attention, b8 s128 h12
+       copy       plain device copy of 256 MiB (counter calibration: reads and
+                  writes exactly 268435456 bytes each)
+Each call goes through the C-ABI via the C++ driver's timing helpers.
+"""
+import ctypes
+import importlib
+import os
+import sys
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path.insert(0, ROOT)
+
+
+def main():
+    what = sys.argv[1]
+    iters = int(sys.argv[2]) if len(sys.argv) > 2 else 20
+    rt = importlib.import_module("hands-on-mlir_amd.hom_runtime")
+    drv, lib = rt.load_driver(), rt.load_runtime()
+    idx, sk = ctypes.c_int64(), ctypes.c_int32()
+    if what == "gemm1":
+        lib.homGemmSelect(1024, 3072, 768, 2, ctypes.byref(idx), ctypes.byref(sk))
+        ms = drv.homTimeGemm(1024, 3072, 768, 2, 1, idx.value + 1, sk.value, iters, 3)
+        print(f"gemm1 {lib.homGemmManifestName(idx.value).decode()} splitK {sk.value}: {ms * 1e3:.2f} us")
+    elif what == "gemm5":
+        lib.homGemmSelect(16384, 1024, 4096, 0, ctypes.byref(idx), ctypes.byref(sk))
+        ms = drv.homTimeGemm(16384, 1024, 4096, 0, 0, idx.value + 1, sk.value, iters, 3)
+        print(f"gemm5 {lib.homGemmManifestName(idx.value).decode()} splitK {sk.value}: {ms * 1e3:.2f} us")
+    elif what == "layernorm":
+        print(f"layernorm 16384x1024: {drv.homTimeLayernorm(16384, 1024, 0, iters, 3) * 1e3:.2f} us")
+    elif what == "attention":
+        lens = (ctypes.c_int32 * 8)(83, 128, 57, 101, 32, 120, 64, 99)
+        print(f"attention b8 s128 h12: {drv.homTimeAttention(8, 128, 12, lens, iters, 3) * 1e3:.2f} us")
+    elif what == "copy":
+        import torch
+        src = torch.ones(128 * 1024 * 1024, dtype=torch.float16, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(iters):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print("copy 268435456 bytes x", iters)
+    else:
+        sys.exit(__doc__)
+
+
+if __name__ == "__main__":
+    main()
