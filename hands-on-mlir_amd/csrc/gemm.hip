@@ -44,9 +44,20 @@
 #include "kernels.h"
 
 #include <type_traits>
+#include <utility>
 
 namespace hom {
 namespace {
+
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>), unrolled.
+template <class F, int... I>
+__device__ __forceinline__ void staticForImpl(F &&f,
+                                              std::integer_sequence<int, I...>) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, class F> __device__ __forceinline__ void staticFor(F &&f) {
+  staticForImpl(f, std::make_integer_sequence<int, N>{});
+}
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef _Float16 half4 __attribute__((ext_vector_type(4)));
@@ -74,13 +85,31 @@ struct GemmParams {
   int kTilesPerSlice;
 };
 
+// GELU(x) = 0.5 x (1 + erf(x / sqrt 2)) with erfc(|z|) = t (a1 + t (a2 + ...))
+// exp(-z^2), t = 1 / (1 + p |z|) (Abramowitz & Stegun 7.1.26, |error| <=
+// 1.5e-7 on erfc, far below half a unit of the fp16 result):
+//   x >= 0: 1 + erf(z) = 2 - erfc(z);   x < 0: 1 + erf(z) = erfc(|z|)
+// so GELU(x) = max(x, 0) - 0.5 |x| erfc(|z|), with no cancellation on the
+// negative side.  A third of the instructions of the library erff.
 __device__ __forceinline__ float geluErf(float x) {
-  return 0.5f * x * (1.0f + erff(x * 0.70710678118654752440f));
+  const float ax = fabsf(x);
+  const float t =
+      __builtin_amdgcn_rcpf(fmaf(0.3275911f * 0.70710678118654752440f, ax, 1.0f));
+  float poly = fmaf(1.061405429f, t, -1.453152027f);
+  poly = fmaf(poly, t, 1.421413741f);
+  poly = fmaf(poly, t, -0.284496736f);
+  poly = fmaf(poly, t, 0.254829592f);
+  // exp(-x^2 / 2) = exp2(-x^2 * 0.5 * log2(e))
+  const float e = __builtin_amdgcn_exp2f(ax * ax * -0.72134752044448170368f);
+  const float erfcAbs = poly * t * e;
+  return fmaf(-0.5f * ax, erfcAbs, fmaxf(x, 0.0f));
 }
 // 0.5 x (1 + tanh(u)) == x / (1 + exp(-2u)), u = sqrt(2/pi) (x + 0.044715 x^3)
 __device__ __forceinline__ float geluTanh(float x) {
   const float u = 0.7978845608028654f * (x + 0.044715f * x * x * x);
-  return x / (1.0f + __expf(-2.0f * u));
+  // exp(-2u) = exp2(-2 log2(e) u); large negative x gives x * rcp(inf) = -0
+  const float e = __builtin_amdgcn_exp2f(u * -2.88539008177792681472f);
+  return x * __builtin_amdgcn_rcpf(1.0f + e);
 }
 
 template <int EPI> __device__ __forceinline__ float activate(float v) {
@@ -166,6 +195,72 @@ __device__ __forceinline__ void epilogueStore(const GemmParams &p,
             }
           }
         }
+      }
+    }
+  }
+}
+
+// Same result as epilogueStore for 8-aligned problems, with full-width memory
+// accesses: each wavefront turns its accumulators around through a private LDS
+// strip (32 rows x WTN fp32, rows padded by 16 bytes), so that a lane ends up
+// with 8 consecutive columns of one row and reads C / writes D 16 bytes at a
+// time, a row segment of WTN halves per WTN/8 lanes.  In accumulator order a
+// store instruction scatters 16-byte pieces over 32 rows, which costs more
+// than a microsecond on a 1024 x 3072 output.  `smem` is the main loop's LDS;
+// the barrier makes sure no wavefront still reads operands from it.
+template <int MI, int NI, int WTM, int WTN, int EPI>
+__device__ __forceinline__ void
+epilogueStoreLds(const GemmParams &p, float16v (&acc)[MI][NI], int m0, int n0,
+                 int waveM, int waveN, int lane, int wave,
+                 unsigned char *smem) {
+  constexpr int ROW_B = WTN * 4 + 16;
+  constexpr int LPR = WTN / 8;  // lanes per row on the way out
+  constexpr int RPP = 64 / LPR; // rows per pass
+  unsigned char *mine = smem + wave * (32 * ROW_B);
+  const int l32 = lane % 32, kb = lane / 32;
+  const bool useC = p.beta != 0.f;
+  const int rr = lane / LPR, cc = (lane % LPR) * 8;
+  const int n = n0 + waveN * WTN + cc;
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < MI; i++) {
+#pragma unroll
+    for (int j = 0; j < NI; j++)
+#pragma unroll
+      for (int g = 0; g < 4; g++) {
+        float4v v;
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+          v[e] = acc[i][j][g * 4 + e];
+        *reinterpret_cast<float4v *>(mine + l32 * ROW_B +
+                                     (j * 32 + g * 8 + kb * 4) * 4) = v;
+      }
+#pragma unroll
+    for (int pass = 0; pass < 32 / RPP; pass++) {
+      const int r = pass * RPP + rr;
+      const float4v lo =
+          *reinterpret_cast<const float4v *>(mine + r * ROW_B + cc * 4);
+      const float4v hi =
+          *reinterpret_cast<const float4v *>(mine + r * ROW_B + cc * 4 + 16);
+      const int m = m0 + waveM * WTM + i * 32 + r;
+      if (m < p.M && n < p.N) {
+        float c[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        if (useC) {
+          const half8 cv = *reinterpret_cast<const half8 *>(
+              p.C + int64_t(m % p.cRowPeriod) * p.ldc + n);
+#pragma unroll
+          for (int e = 0; e < 8; e++)
+            c[e] = float(cv[e]);
+        }
+        half8 o;
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+          float v = p.alpha * (e < 4 ? lo[e] : hi[e - 4]);
+          if (useC)
+            v += p.beta * c[e];
+          o[e] = _Float16(activate<EPI>(v));
+        }
+        *reinterpret_cast<half8 *>(p.D + int64_t(m) * p.ldd + n) = o;
       }
     }
   }
@@ -484,7 +579,10 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmDmaKernel(GemmParams p) {
     storePartial<MI, NI, THREADS>(p, acc, tile, slice, numSlices, tid);
     return;
   }
-  epilogueStore<MI, NI, WTM, WTN, EPI, 8>(p, acc, m0, n0, waveM, waveN, lane);
+  static_assert(WM * WN * 32 * (WTN * 4 + 16) <= 2 * STAGE_BYTES,
+                "epilogue strips must fit the main loop's LDS");
+  epilogueStoreLds<MI, NI, WTM, WTN, EPI>(p, acc, m0, n0, waveM, waveN, lane,
+                                          wave, smem);
 #endif
 }
 
@@ -495,8 +593,9 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmDmaKernel(GemmParams p) {
 // The vector memory path into registers sustains several times the bandwidth
 // of the LDS-DMA path on this chip, which matters once a CU streams more than
 // ~16 bytes per clock (large tiles, or several workgroups per CU).
-template <int BM, int BN, int WM, int WN, int DIST, int EPI, bool B_NK>
+template <int BM, int BN, int WM, int WN, int DIST, int FB, int EPI, bool B_NK>
 __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(GemmParams p) {
+  static_assert(DIST >= 1 && (FB == 1 || FB == 2), "unsupported pipeline shape");
   constexpr int BK = 64;
   constexpr int THREADS = WM * WN * kWave;
   constexpr int WTM = BM / WM, WTN = BN / WN;
@@ -529,22 +628,41 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(GemmParams p) {
   if (ktEnd > kTiles)
     ktEnd = kTiles;
 
-  // ---- global sources: a uniform tile base plus a constant 32-bit element
-  // offset per thread.  Rows / columns past the edge are clamped to the last
-  // valid one: what they fetch only reaches outputs that are never stored, so
-  // full slabs need no predication (the K tail does).
+  // ---- global sources ----
+  // Buffer loads from descriptors based at this tile's first row (A) / first
+  // row or column block (B): a constant 32-bit byte offset per thread plus a
+  // scalar offset per slab.  Rows / columns past the edge are clamped to the
+  // last valid one: what they fetch only reaches outputs that are never
+  // stored.  Vectors at or past kEnd (the K tail, and whole slabs requested
+  // beyond this slice) get an offset outside the descriptor and read as zero
+  // without touching memory, so every slab issues the same number of loads
+  // and the compiler's outstanding-load counts are exact -- a branch around a
+  // load makes it wait for everything in flight and defeats the pipeline.
+  constexpr uint32_t kOob = 0x80000000u;
+  auto clampBytes = [](int64_t b) -> int32_t {
+    return b > 0x7fffffffLL ? 0x7fffffff : (b < 0 ? 0 : int32_t(b));
+  };
   const _Float16 *aTile = p.A + int64_t(m0) * p.lda;
+  const auto rsrcA = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<_Float16 *>(aTile), 0,
+      clampBytes(int64_t(p.M - m0) * p.lda * 2), 0x00020000);
   const _Float16 *bTile = B_NK ? p.B + int64_t(n0) * p.ldb : p.B + n0;
+  const auto rsrcB = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<_Float16 *>(bTile), 0,
+      clampBytes(B_NK ? int64_t(p.N - n0) * p.ldb * 2
+                      : (int64_t(p.K) * p.ldb - n0) * 2),
+      0x00020000);
+  const int kEnd = ktEnd * BK < p.K ? ktEnd * BK : p.K;
   uint32_t aOff[A_PER_T], bOff[B_PER_T];
   int aDst[A_PER_T], bDst[B_PER_T];
-  int aK[A_PER_T], bK[B_PER_T]; // k position inside the slab (for the tail)
+  int aK[A_PER_T], bK[B_PER_T]; // k position inside the slab
 #pragma unroll
   for (int i = 0; i < A_PER_T; i++) {
     const int v = tid + i * THREADS;
     const int r = v / 8, c = v % 8;
     const int rr = m0 + r < p.M ? r : p.M - 1 - m0;
     aK[i] = c * 8;
-    aOff[i] = uint32_t(rr) * uint32_t(p.lda) + c * 8;
+    aOff[i] = (uint32_t(rr) * uint32_t(p.lda) + c * 8) * 2u;
     aDst[i] = r * 128 + swzK(r, c) * 16;
   }
 #pragma unroll
@@ -554,48 +672,32 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(GemmParams p) {
     if (B_NK) {
       const int rr = n0 + r < p.N ? r : p.N - 1 - n0;
       bK[i] = c * 8;
-      bOff[i] = uint32_t(rr) * uint32_t(p.ldb) + c * 8;
+      bOff[i] = (uint32_t(rr) * uint32_t(p.ldb) + c * 8) * 2u;
       bDst[i] = r * 128 + swzK(r, c) * 16;
     } else {
       const int cc = n0 + c * 8 < p.N ? c * 8 : p.N - 8 - n0;
       bK[i] = r;
-      bOff[i] = uint32_t(r) * uint32_t(p.ldb) + cc;
+      bOff[i] = (uint32_t(r) * uint32_t(p.ldb) + cc) * 2u;
       bDst[i] = r * B_ROW_BYTES + swzN<BN>(r, c / 4) * 64 + (c % 4) * 16;
     }
   }
 
   half8 regA[DIST][A_PER_T], regB[DIST][B_PER_T];
-  auto zero8 = []() {
-    half8 z;
-#pragma unroll
-    for (int e = 0; e < 8; e++)
-      z[e] = _Float16(0);
-    return z;
-  };
   auto loadGlobal = [&](int kt, auto setC) {
     constexpr int S = decltype(setC)::value;
     const int k0 = kt * BK;
-    const _Float16 *aSlab = aTile + k0;
-    const _Float16 *bSlab = B_NK ? bTile + k0 : bTile + int64_t(k0) * p.ldb;
-    if (k0 + BK <= p.K) {
+    const uint32_t sA = uint32_t(k0) * 2u;
+    const uint32_t sB = B_NK ? sA : uint32_t(k0) * uint32_t(p.ldb) * 2u;
 #pragma unroll
-      for (int i = 0; i < A_PER_T; i++)
-        regA[S][i] = *reinterpret_cast<const half8 *>(aSlab + aOff[i]);
+    for (int i = 0; i < A_PER_T; i++)
+      regA[S][i] = __builtin_bit_cast(
+          half8, __builtin_amdgcn_raw_buffer_load_b128(
+                     rsrcA, k0 + aK[i] < kEnd ? aOff[i] : kOob, sA, 0));
 #pragma unroll
-      for (int i = 0; i < B_PER_T; i++)
-        regB[S][i] = *reinterpret_cast<const half8 *>(bSlab + bOff[i]);
-    } else {
-#pragma unroll
-      for (int i = 0; i < A_PER_T; i++)
-        regA[S][i] = k0 + aK[i] < p.K
-                      ? *reinterpret_cast<const half8 *>(aSlab + aOff[i])
-                      : zero8();
-#pragma unroll
-      for (int i = 0; i < B_PER_T; i++)
-        regB[S][i] = k0 + bK[i] < p.K
-                      ? *reinterpret_cast<const half8 *>(bSlab + bOff[i])
-                      : zero8();
-    }
+    for (int i = 0; i < B_PER_T; i++)
+      regB[S][i] = __builtin_bit_cast(
+          half8, __builtin_amdgcn_raw_buffer_load_b128(
+                     rsrcB, k0 + bK[i] < kEnd ? bOff[i] : kOob, sB, 0));
   };
   auto storeLds = [&](int stage, auto setC) {
     constexpr int S = decltype(setC)::value;
@@ -644,107 +746,205 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(GemmParams p) {
                 swzN<BN>(trRow, group) * 64 + trCol * 2;
   }
 
-  auto loadFrags = [&](int stage, int kk, half8 (&fa)[MI], half8 (&fb)[NI]) {
+  // One fragment per call: unit u < MI is A block u, the rest are B blocks.
+  auto loadFragUnit = [&](int stage, int kk, half8 (&fa)[MI], half8 (&fb)[NI],
+                          auto uC) {
+    constexpr int U = decltype(uC)::value;
     const unsigned char *st = smem + stage * STAGE_BYTES;
-#pragma unroll
-    for (int i = 0; i < MI; i++)
-      fa[i] = *reinterpret_cast<const half8 *>(st + aFrag[kk] + i * 32 * 128);
-    if (B_NK) {
-#pragma unroll
-      for (int j = 0; j < NI; j++)
-        fb[j] = *reinterpret_cast<const half8 *>(st + bFragK[kk] + j * 32 * 128);
+    if constexpr (U < MI) {
+      fa[U] = *reinterpret_cast<const half8 *>(st + aFrag[kk] + U * 32 * 128);
+    } else if constexpr (B_NK) {
+      constexpr int j = U - MI;
+      fb[j] = *reinterpret_cast<const half8 *>(st + bFragK[kk] + j * 32 * 128);
     } else {
+      constexpr int j = U - MI;
+      short4v t[2];
 #pragma unroll
-      for (int j = 0; j < NI; j++) {
-        short4v t[2];
+      for (int h = 0; h < 2; h++)
+        t[h] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (__attribute__((address_space(3))) short4v *)(
+                st + bFragN[j] + (kk * 16 + h * 4) * B_ROW_BYTES));
+      typedef short short8v __attribute__((ext_vector_type(8)));
+      short8v both;
 #pragma unroll
-        for (int h = 0; h < 2; h++)
-          t[h] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-              (__attribute__((address_space(3))) short4v *)(
-                  st + bFragN[j] + (kk * 16 + h * 4) * B_ROW_BYTES));
-        typedef short short8v __attribute__((ext_vector_type(8)));
-        short8v both;
-#pragma unroll
-        for (int e = 0; e < 4; e++) {
-          both[e] = t[0][e];
-          both[4 + e] = t[1][e];
-        }
-        fb[j] = __builtin_bit_cast(half8, both);
+      for (int e = 0; e < 4; e++) {
+        both[e] = t[0][e];
+        both[4 + e] = t[1][e];
       }
+      fb[j] = __builtin_bit_cast(half8, both);
     }
   };
-  auto mfmaStep = [&](half8 (&fa)[MI], half8 (&fb)[NI]) {
-#pragma unroll
-    for (int i = 0; i < MI; i++)
-#pragma unroll
-      for (int j = 0; j < NI; j++)
-        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[j], fa[i],
-                                                           acc[i][j], 0, 0, 0);
+  auto loadFrags = [&](int stage, int kk, half8 (&fa)[MI], half8 (&fb)[NI]) {
+    staticFor<MI + NI>([&](auto uC) { loadFragUnit(stage, kk, fa, fb, uC); });
   };
 
   // ---- main loop ----
-  // LDS holds slab i (buffer i & 1); slab i+1 sits in registers (or is on its way
-  // there) and is written to the other buffer after the third k step; with
-  // DIST == 2 the register set that was just written out is refilled with slab
-  // i+3 at once, so two slabs of global loads are in flight per workgroup -- on
-  // this chip one slab per CU in flight is not enough to cover memory latency.
+  // LDS holds slab i (buffer i & 1); slabs i+1 .. i+DIST sit in registers or are
+  // on their way there, slab s in register set s % DIST.  While slab i is
+  // multiplied, slab i+1 moves from its register set to the other LDS buffer
+  // one 16-byte vector at a time, and each vector's registers are refilled
+  // with slab i+1+DIST right behind the LDS write.  These LDS writes and global
+  // loads are spread between the MFMAs of the first KSTEPS-1 k steps
+  // (scheduling barriers pin the order): issued as one burst they fill the
+  // memory pipelines' queues, the wavefront blocks on issue, and with both
+  // wavefronts of a SIMD in the same phase the matrix core idles for as long as
+  // the burst takes to drain.  The loop is unrolled DIST times to keep the
+  // register-set index a compile-time constant.
   // The barrier is a bare s_barrier behind an LDS-only wait: a fence here would
   // drain the global loads that were just issued.
-  using Set0 = std::integral_constant<int, 0>;
-  using Set1 = std::integral_constant<int, DIST - 1>;
-  half8 fa[2][MI], fb[2][NI];
+  // FB == 2 fetches the fragments of k step kk+1 before the MFMAs of step kk
+  // (two fragment sets); FB == 1 keeps one set and relies on the other
+  // wavefronts of the SIMD to cover the LDS latency, which frees registers for a
+  // deeper global pipeline on the largest tiles.
+  constexpr int NV = A_PER_T + B_PER_T; // vectors per thread and slab
+  constexpr int NM = MI * NI;           // MFMAs per wavefront and k step
+  constexpr int ST_STEPS = KSTEPS - 1;  // k steps that carry staging work
+  half8 fa[FB][MI], fb[FB][NI];
   const int nk = ktEnd - ktBegin;
-  auto slab = [&](int i, auto setC) {
+  // Moves vector v of register set S to LDS and refills it from slab kt.
+  auto stageVec = [&](int stage, int kt, auto setC, auto vC) {
+    constexpr int S = decltype(setC)::value;
+    constexpr int V = decltype(vC)::value;
+    unsigned char *sA = smem + stage * STAGE_BYTES;
+    unsigned char *sB = sA + A_BYTES;
+    const int k0 = kt * BK;
+    if constexpr (V < A_PER_T) {
+      *reinterpret_cast<half8 *>(sA + aDst[V]) = regA[S][V];
+      regA[S][V] = __builtin_bit_cast(
+          half8, __builtin_amdgcn_raw_buffer_load_b128(
+                     rsrcA, k0 + aK[V] < kEnd ? aOff[V] : kOob,
+                     uint32_t(k0) * 2u, 0));
+    } else {
+      constexpr int W = V - A_PER_T;
+      *reinterpret_cast<half8 *>(sB + bDst[W]) = regB[S][W];
+      regB[S][W] = __builtin_bit_cast(
+          half8,
+          __builtin_amdgcn_raw_buffer_load_b128(
+              rsrcB, k0 + bK[W] < kEnd ? bOff[W] : kOob,
+              B_NK ? uint32_t(k0) * 2u : uint32_t(k0) * uint32_t(p.ldb) * 2u,
+              0));
+    }
+  };
+  // The MFMAs of one k step on fragments (a, b).  Spread between them: the
+  // fragment reads of another k step (rdStage, rdKk) into (na, nb) when RD, and
+  // the staging vectors [V0, V1) when stageOn.  Memory operation q of n goes in
+  // front of MFMA q * NM / n.
+  auto mfmaMixed = [&](half8 (&a)[MI], half8 (&b)[NI], half8 (&na)[MI],
+                       half8 (&nb)[NI], int rdStage, int rdKk, auto rdC,
+                       int stStage, int kt, bool stageOn, auto setC, auto v0C,
+                       auto v1C) {
+    constexpr bool RD = decltype(rdC)::value;
+    constexpr int V0 = decltype(v0C)::value, V1 = decltype(v1C)::value;
+    constexpr int NR = RD ? MI + NI : 0;
+    constexpr int N = NR + (V1 - V0);
+    staticFor<NM>([&](auto mC) {
+      constexpr int m = decltype(mC)::value;
+      if constexpr (N > 0) {
+        staticFor<N>([&](auto qC) {
+          constexpr int q = decltype(qC)::value;
+          if constexpr (q * NM / N == m) {
+            __builtin_amdgcn_sched_barrier(0);
+            if constexpr (q < NR) {
+              loadFragUnit(rdStage, rdKk, na, nb,
+                           std::integral_constant<int, (q < NR ? q : 0)>{});
+            } else {
+              if (stageOn)
+                stageVec(stStage, kt, setC,
+                         std::integral_constant<int, V0 + q - NR>{});
+            }
+            __builtin_amdgcn_sched_barrier(0);
+          }
+        });
+      }
+      acc[m / NI][m % NI] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+          b[m % NI], a[m / NI], acc[m / NI][m % NI], 0, 0, 0);
+    });
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  // tailC: the slab may be the last one (then nothing follows it); the
+  // steady-state loop knows it is not and runs without branches.
+  auto slab = [&](int i, auto setC, auto tailC) {
+    constexpr bool kTail = decltype(tailC)::value;
     const int cur = i & 1;
-    const bool more = i + 1 < nk;
-    if (DIST == 1 && more)
-      loadGlobal(ktBegin + i + 1, setC);
-#pragma unroll
-    for (int kk = 0; kk < KSTEPS - 1; kk++) {
-      loadFrags(cur, kk + 1, fa[(kk + 1) & 1], fb[(kk + 1) & 1]);
-      mfmaStep(fa[kk & 1], fb[kk & 1]);
-    }
-    if (more) {
-      // The other buffer was last read before the previous barrier, so it can
-      // be overwritten now; after this barrier every wavefront has its last
-      // fragments of slab i in registers and slab i+1 is visible.
-      storeLds(cur ^ 1, setC);
-      if (DIST == 2 && i + 3 < nk)
-        loadGlobal(ktBegin + i + 3, setC);
-      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-      loadFrags(cur ^ 1, 0, fa[0], fb[0]);
-    }
-    mfmaStep(fa[(KSTEPS - 1) & 1], fb[(KSTEPS - 1) & 1]);
+    const bool more = !kTail || i + 1 < nk;
+    const int ktNext = ktBegin + i + 1 + DIST;
+    staticFor<KSTEPS>([&](auto kkC) {
+      constexpr int kk = decltype(kkC)::value;
+      constexpr int V0 = kk < ST_STEPS ? kk * NV / ST_STEPS : NV;
+      constexpr int V1 = kk < ST_STEPS ? (kk + 1) * NV / ST_STEPS : NV;
+      using V0C = std::integral_constant<int, V0>;
+      using V1C = std::integral_constant<int, V1>;
+      constexpr int cs = kk % FB, ns = (kk + 1) % FB;
+      if constexpr (kk < KSTEPS - 1) {
+        if constexpr (FB == 2) {
+          mfmaMixed(fa[cs], fb[cs], fa[ns], fb[ns], cur, kk + 1,
+                    std::true_type{}, cur ^ 1, ktNext, more, setC, V0C{},
+                    V1C{});
+        } else {
+          if (kk > 0)
+            loadFrags(cur, kk, fa[0], fb[0]);
+          __builtin_amdgcn_sched_barrier(0);
+          mfmaMixed(fa[0], fb[0], fa[0], fb[0], 0, 0, std::false_type{},
+                    cur ^ 1, ktNext, more, setC, V0C{}, V1C{});
+        }
+      } else {
+        if constexpr (FB == 1) {
+          loadFrags(cur, kk, fa[0], fb[0]);
+          mfmaMixed(fa[0], fb[0], fa[0], fb[0], 0, 0, std::false_type{}, 0, 0,
+                    false, setC, V0C{}, V1C{});
+        }
+        if (more) {
+          // Every wavefront has its last fragments of slab i in registers and
+          // slab i+1 is complete in the other buffer after this barrier.
+          asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        }
+        if constexpr (FB == 2) {
+          // ns == 0: the first fragments of slab i+1 arrive under these MFMAs
+          if (more)
+            mfmaMixed(fa[cs], fb[cs], fa[ns], fb[ns], cur ^ 1, 0,
+                      std::true_type{}, 0, 0, false, setC, V0C{}, V1C{});
+          else
+            mfmaMixed(fa[cs], fb[cs], fa[ns], fb[ns], 0, 0, std::false_type{},
+                      0, 0, false, setC, V0C{}, V1C{});
+        } else if (more) {
+          loadFrags(cur ^ 1, 0, fa[0], fb[0]);
+        }
+      }
+    });
   };
   if (nk > 0) {
-    loadGlobal(ktBegin, Set0{});
-    storeLds(0, Set0{});
-    if (DIST == 2) {
-      if (nk > 1)
-        loadGlobal(ktBegin + 1, Set1{});
-      if (nk > 2)
-        loadGlobal(ktBegin + 2, Set0{});
-    }
+    staticFor<DIST>(
+        [&](auto d) { loadGlobal(ktBegin + decltype(d)::value, d); });
+    storeLds(0, std::integral_constant<int, 0>{});
+    loadGlobal(ktBegin + DIST, std::integral_constant<int, 0>{});
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
     loadFrags(0, 0, fa[0], fb[0]);
-    if (DIST == 1) {
-      for (int i = 0; i < nk; i++)
-        slab(i, Set0{});
-    } else {
-      // slab i+1 lives in register set (i+1) & 1
-      for (int i = 0; i < nk; i += 2) {
-        slab(i, Set1{});
-        if (i + 1 < nk)
-          slab(i + 1, Set0{});
-      }
+    int i = 0;
+    for (; i + DIST < nk; i += DIST) {
+      staticFor<DIST>([&](auto d) {
+        constexpr int D = decltype(d)::value;
+        slab(i + D, std::integral_constant<int, (D + 1) % DIST>{},
+             std::false_type{});
+      });
     }
+    bool go = true;
+    staticFor<DIST>([&](auto d) {
+      constexpr int D = decltype(d)::value;
+      go = go && i + D < nk;
+      if (go)
+        slab(i + D, std::integral_constant<int, (D + 1) % DIST>{},
+             std::true_type{});
+    });
   }
 
   if (numSlices > 1) {
     storePartial<MI, NI, THREADS>(p, acc, tile, slice, numSlices, tid);
     return;
   }
-  epilogueStore<MI, NI, WTM, WTN, EPI, 8>(p, acc, m0, n0, waveM, waveN, lane);
+  static_assert(WM * WN * 32 * (WTN * 4 + 16) <= 2 * STAGE_BYTES,
+                "epilogue strips must fit the main loop's LDS");
+  epilogueStoreLds<MI, NI, WTM, WTN, EPI>(p, acc, m0, n0, waveM, waveN, lane,
+                                          wave, smem);
 }
 
 // ================================================================== staged ==
@@ -1135,14 +1335,21 @@ Status launchDma(const GemmProblem &pr, hipStream_t s) {
   return Status::kSuccess;
 }
 
-template <int BM, int BN, int WM, int WN, int DIST, int EPI, bool B_NK>
+template <int BM, int BN, int WM, int WN, int DIST, int FB, int EPI, bool B_NK>
 Status launchPipe(const GemmProblem &pr, hipStream_t s) {
   constexpr int SMEM = 2 * (BM + BN) * 64 * 2;
   LaunchPlan plan;
   Status st = planLaunch<BM, BN, 64>(pr, &plan);
   if (st != Status::kSuccess)
     return st;
-  auto kernel = gemmPipeKernel<BM, BN, WM, WN, DIST, EPI, B_NK>;
+  // 32-bit buffer offsets: a row-major B slab is addressed from the matrix base.
+  HOM_CHECK_RET(B_NK || pr.K * pr.ldb * 2 < (int64_t(1) << 31),
+                Status::kInvalidArgument,
+                "gemm: B larger than 2 GiB is not supported by this kernel");
+  HOM_CHECK_RET((int64_t(BM) * pr.lda + pr.K) * 2 < (int64_t(1) << 31) &&
+                    (int64_t(BN) * pr.ldb + pr.K) * 2 < (int64_t(1) << 31),
+                Status::kInvalidArgument, "gemm: leading dimension too large");
+  auto kernel = gemmPipeKernel<BM, BN, WM, WN, DIST, FB, EPI, B_NK>;
   static bool attrSet = false;
   st = allowLds(kernel, SMEM, &attrSet);
   if (st != Status::kSuccess)
@@ -1183,19 +1390,26 @@ struct KernelEntry {
       HOM_DMA_ENTRY(BM, BN, WM, WN, NS, Epilogue::kGeluTanh, "gelutanh", 1)
 
 // "r<d>" after the LDS stage count marks the register-staged pipeline with d
-// slabs of global loads in flight.
-#define HOM_PIPE_ENTRY(BM, BN, WM, WN, DIST, EPI_ENUM, EPI_STR, ACT)           \
+// slabs of global loads in flight; a trailing "s" a single fragment set.
+#define HOM_PIPE_ENTRY(BM, BN, WM, WN, DIST, FB, FBS, EPI_ENUM, EPI_STR, ACT)  \
   {                                                                            \
-    {"hom_gfx950_mfma_f16_s32x32x16gemm_f16_" #BM "x" #BN "_64x2r" #DIST       \
+    {"hom_gfx950_mfma_f16_s32x32x16gemm_f16_" #BM "x" #BN "_64x2r" #DIST FBS   \
      "_w" #WM "x" #WN "_nn_align8_" EPI_STR,                                   \
      BM, BN, 64, WM, WN, 8, ACT, EPI_ENUM},                                    \
-        launchPipe<BM, BN, WM, WN, DIST, int(EPI_ENUM), false>,                \
-        launchPipe<BM, BN, WM, WN, DIST, int(EPI_ENUM), true>                  \
+        launchPipe<BM, BN, WM, WN, DIST, FB, int(EPI_ENUM), false>,            \
+        launchPipe<BM, BN, WM, WN, DIST, FB, int(EPI_ENUM), true>              \
   }
+#define HOM_PIPE_TILE_FB(BM, BN, WM, WN, DIST, FB, FBS)                        \
+  HOM_PIPE_ENTRY(BM, BN, WM, WN, DIST, FB, FBS, Epilogue::kLinear, "linear",   \
+                 0),                                                           \
+      HOM_PIPE_ENTRY(BM, BN, WM, WN, DIST, FB, FBS, Epilogue::kGeluErf,        \
+                     "gelu", 1),                                               \
+      HOM_PIPE_ENTRY(BM, BN, WM, WN, DIST, FB, FBS, Epilogue::kGeluTanh,       \
+                     "gelutanh", 1)
 #define HOM_PIPE_TILE(BM, BN, WM, WN, DIST)                                    \
-  HOM_PIPE_ENTRY(BM, BN, WM, WN, DIST, Epilogue::kLinear, "linear", 0),        \
-      HOM_PIPE_ENTRY(BM, BN, WM, WN, DIST, Epilogue::kGeluErf, "gelu", 1),     \
-      HOM_PIPE_ENTRY(BM, BN, WM, WN, DIST, Epilogue::kGeluTanh, "gelutanh", 1)
+  HOM_PIPE_TILE_FB(BM, BN, WM, WN, DIST, 2, "")
+#define HOM_PIPE_TILE_S(BM, BN, WM, WN, DIST)                                  \
+  HOM_PIPE_TILE_FB(BM, BN, WM, WN, DIST, 1, "s")
 
 #define HOM_STAGED_ENTRY(BM, BN, BK, WM, WN, EPI_ENUM, EPI_STR, ACT, VEC)      \
   {                                                                            \
@@ -1218,28 +1432,24 @@ const KernelEntry kKernels[] = {
     HOM_DMA_TILE(128, 128, 2, 2, 4),
     HOM_DMA_TILE(64, 64, 2, 2, 4),
     HOM_DMA_TILE(128, 64, 2, 2, 4),
-    HOM_DMA_TILE(64, 128, 2, 2, 4),
-    HOM_DMA_TILE(256, 128, 2, 2, 3),
-    HOM_DMA_TILE(128, 256, 2, 2, 3),
-    HOM_DMA_TILE(256, 256, 2, 2, 2),
-    HOM_DMA_TILE(128, 128, 2, 2, 2),
     HOM_DMA_TILE(64, 64, 2, 2, 8),
-    HOM_DMA_TILE(128, 128, 2, 4, 4),
-    HOM_DMA_TILE(256, 128, 4, 2, 3),
     HOM_DMA_TILE(256, 256, 2, 4, 2),
-    HOM_DMA_TILE(128, 256, 2, 4, 3),
-    HOM_PIPE_TILE(64, 64, 2, 2, 1),
-    HOM_PIPE_TILE(128, 64, 2, 2, 1),
-    HOM_PIPE_TILE(64, 128, 2, 2, 1),
-    HOM_PIPE_TILE(128, 128, 2, 2, 1),
-    HOM_PIPE_TILE(128, 128, 2, 4, 1),
-    HOM_PIPE_TILE(256, 256, 2, 4, 1),
     HOM_PIPE_TILE(64, 64, 2, 2, 2),
+    HOM_PIPE_TILE(64, 64, 2, 2, 4),
+    HOM_PIPE_TILE(128, 64, 2, 2, 2),
+    HOM_PIPE_TILE(128, 64, 2, 2, 4),
+    HOM_PIPE_TILE(64, 128, 2, 2, 2),
+    HOM_PIPE_TILE(64, 128, 2, 2, 4),
     HOM_PIPE_TILE(128, 128, 2, 2, 2),
+    HOM_PIPE_TILE(128, 128, 2, 2, 4),
     HOM_PIPE_TILE(128, 128, 2, 4, 2),
+    HOM_PIPE_TILE(128, 128, 2, 4, 4),
     HOM_PIPE_TILE(256, 128, 4, 2, 2),
+    HOM_PIPE_TILE(256, 128, 4, 2, 3),
     HOM_PIPE_TILE(128, 256, 2, 4, 2),
-    HOM_PIPE_TILE(256, 256, 2, 4, 2),
+    HOM_PIPE_TILE(128, 256, 2, 4, 3),
+    HOM_PIPE_TILE(256, 256, 2, 4, 1),
+    HOM_PIPE_TILE(256, 256, 2, 2, 1),
     HOM_STAGED_TILE(128, 128, 32, 2, 2, 8),
     HOM_STAGED_TILE(64, 64, 64, 2, 2, 8),
     HOM_STAGED_TILE(64, 64, 32, 2, 2, 1),
@@ -1271,8 +1481,8 @@ Status launchGemm(int idx, const GemmProblem &p, hipStream_t s) {
   if (k.info.alignment == 8) {
     // What CUTLASS's can_implement() rejects: misaligned leading dimensions.
     const bool ok = p.N % 8 == 0 && p.K % 8 == 0 && p.lda % 8 == 0 &&
-                    p.ldb % 8 == 0 && p.ldd % 4 == 0 &&
-                    (p.beta == 0.f || p.ldc % 4 == 0) && aligned16(p.A) &&
+                    p.ldb % 8 == 0 && p.ldd % 8 == 0 &&
+                    (p.beta == 0.f || p.ldc % 8 == 0) && aligned16(p.A) &&
                     aligned16(p.B) && aligned16(p.D) &&
                     (p.beta == 0.f || aligned16(p.C));
     HOM_CHECK_RET(ok, Status::kInvalidArgument,
