@@ -75,6 +75,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-large", action="store_true", help="skip the BERT-large b32 x s512 encoder timing")
     ap.add_argument("--eager", action="store_true", help="launch every call instead of replaying a HIP graph")
     ap.add_argument("--gemm-mode", type=int, default=1,
                     help="0 nvteGemmF16 path, 1 cutlassGemmF16 + tuned table, 2 + live autotune")
@@ -152,6 +153,21 @@ def main():
         tf = 2.0 * m * n * k / (t * 1e-3) / 1e12
         kernels[tag] = {"us": t * 1e3, "TFLOP/s": tf, "frac_mfma": tf / PEAK_FP16_TFLOPS,
                         "kernel": names[idx.value + 1], "splitK": sk.value}
+
+    if not args.no_large:
+        # configs[4]: BERT-large encoder end to end (reported beside the headline, not as `value`)
+        big = synth.bert_encoder(layers=24, hidden=1024, heads=16, ffn=4096, bs=32, seq=512, config=41)
+        enc = bert.BertEncoder(24, 1024, 16, 4096, 32, 512, big["dims"]["vocab"],
+                               gemm_mode=args.gemm_mode, gelu_form="erf")
+        enc.load(big)
+        enc.set_inputs(ids=big["ids"], mask=big["mask"])
+        big_ms = enc.time(20, 3, graph=not args.eager)
+        enc.close()
+        attn_flops = 4 * 16 * 64 * float(sum(int(n) ** 2 for n in big["lens"]))
+        big_flops = 24 * (2.0 * 16384 * 1024 * (3 * 1024 + 1024 + 2 * 4096) + attn_flops)
+        kernels["bert_large_b32_s512_encoder"] = {"ms": big_ms, "sequences/s": 32 / (big_ms * 1e-3),
+                                                  "TFLOP/s": big_flops / (big_ms * 1e-3) / 1e12}
+        del big
 
     out = {
         "metric": METRIC, "value": seqs_per_s, "unit": "sequences/s", "n_gpus": 1,

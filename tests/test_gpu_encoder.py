@@ -135,3 +135,99 @@ def test_single_layer_full_width(gpu, oracle, synth):
             print(f"one BERT-base layer (gemm mode {gemm_mode}): norm-wise relative error {rel:.3e}")
         finally:
             enc.close()
+
+
+def ref_flags(got, want32, lens):
+    """The reference driver's own criterion (examples/torch/bert/bert.cu:148-153): an
+    element is wrong only when both its absolute and its relative error exceed 1e-2."""
+    bad = 0
+    for b, n in enumerate(lens):
+        g, w = got[b, :n].astype(np.float64), want32[b, :n].astype(np.float64)
+        err = np.abs(g - w)
+        bad += int(((err > 1e-2) & (err > 1e-2 * np.abs(w))).sum())
+    return bad
+
+
+def test_bert_large_architecture(gpu, oracle, synth):
+    """BERT-large (24 layers, hidden 1024, 16 heads, FFN 4096, seq 512).
+
+    Two sequences against the oracle (a size it finishes in seconds), then the full
+    batch of 32 through size-independent properties: the first two sequences of the
+    big batch reproduce the small run (other tile shapes, same arithmetic), and a
+    sequence's output ignores padding content and its neighbours."""
+    bert = importlib.import_module("hands-on-mlir_amd.bert")
+    big = synth.bert_encoder(layers=24, hidden=1024, heads=16, ffn=4096, bs=32, seq=512, config=41)
+    d = big["dims"]
+    big["lens"][:2] = [512, 301]
+    big["mask"] = synth.mask_from_lengths(big["lens"], 512)
+    small = dict(big, ids=big["ids"][:2].copy(), lens=big["lens"][:2].copy(), mask=big["mask"][:2].copy(),
+                 dims=dict(d, bs=2))
+    enc = bert.BertEncoder(24, 1024, 16, 4096, 2, 512, d["vocab"], gemm_mode=1, gelu_form="erf")
+    try:
+        enc.load(small)
+        enc.set_inputs(ids=small["ids"], mask=small["mask"])
+        enc.capture()
+        enc.replay()
+        got2 = enc.output()
+    finally:
+        enc.close()
+    faithful = oracle_forward(oracle, small, "erf")
+    pure = oracle_forward(oracle, small, "erf", round_intermediates=False)
+
+    def relerr(a, b):
+        e = n = 0.0
+        for s, ln in enumerate(small["lens"]):
+            x, y = a[s, :ln].astype(np.float64), b[s, :ln].astype(np.float64)
+            e += ((x - y) ** 2).sum()
+            n += (y ** 2).sum()
+        return np.sqrt(e / n)
+
+    rel16, rel32 = relerr(got2, faithful), relerr(got2, pure)
+    floor = relerr(faithful.astype(np.float16), pure)
+    print(f"BERT-large b2 s512 norm-wise relative error: {rel16:.3e} vs fp16-faithful oracle, "
+          f"{rel32:.3e} vs fp32 reference (fp16-storage floor {floor:.3e})")
+    # The rounding noise of 24 layers of fp16 storage (rms 1.5e-3 on unit-variance
+    # outputs, the same for the oracle's own fp16 pipeline) puts the reference's 1e-2
+    # threshold at ~7 sigma: allow its tail, 1e-5 of the elements.
+    valid = int(sum(small["lens"])) * 1024
+    flags16, flags32 = ref_flags(got2, faithful, small["lens"]), ref_flags(got2, pure, small["lens"])
+    flags_floor = ref_flags(faithful.astype(np.float16), pure, small["lens"])
+    print(f"elements beyond the reference's criterion: {flags16} vs fp16-faithful oracle, {flags32} vs fp32 "
+          f"reference, {flags_floor} for the oracle's own fp16 pipeline vs fp32 (of {valid})")
+    assert flags16 <= 1e-5 * valid and flags32 <= 1e-5 * valid
+    # 24 layers of decorrelating fp16 rounding noise: sqrt(2) x the 12-layer bound
+    assert rel16 <= 3e-3 and rel32 <= 3e-3
+    assert rel32 <= 1.1 * floor, f"GPU path error {rel32:.3e} exceeds the fp16-storage floor {floor:.3e}"
+
+    enc = bert.BertEncoder(24, 1024, 16, 4096, 32, 512, d["vocab"], gemm_mode=1, gelu_form="erf")
+    try:
+        enc.load(big)
+        enc.set_inputs(ids=big["ids"], mask=big["mask"])
+        enc.capture()
+        enc.replay()
+        got32 = enc.output()
+        assert np.isfinite(got32.astype(np.float32)).all()
+        # same sequences inside the full batch: other tiles and split-K choices, so equal
+        # up to the fp16 rounding noise measured above, not bit for bit
+        assert ref_flags(got32[:2], got2.astype(np.float32), small["lens"]) <= 1e-5 * valid
+        drift = relerr(got32[:2], got2.astype(np.float32))
+        print(f"BERT-large b32 vs b2 on the shared sequences: norm-wise {drift:.3e}")
+        assert drift <= 3e-3
+        # padding content and neighbours do not matter (same launch shapes: bit exact)
+        ids2 = big["ids"].copy()
+        for b, n in enumerate(big["lens"]):
+            ids2[b, n:] = (ids2[b, n:] + 7) % d["vocab"]
+        ids2[2:] = ids2[2:][::-1]
+        mask2 = big["mask"].copy()
+        mask2[2:] = mask2[2:][::-1]
+        enc.set_inputs(ids=ids2, mask=mask2)
+        enc.replay()
+        again = enc.output()
+        for b in (0, 1):
+            n = big["lens"][b]
+            assert np.array_equal(again[b, :n], got32[b, :n])
+        last = 31
+        n = big["lens"][2]
+        assert np.array_equal(again[last, :n], got32[2, :n])
+    finally:
+        enc.close()
