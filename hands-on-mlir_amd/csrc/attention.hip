@@ -62,8 +62,7 @@ __global__ __launch_bounds__(NW *kWave) void bertAttentionKernel(
   const int l32 = lane % 32, hb = lane / 32;
   const int head = blockIdx.y, b = blockIdx.z;
   const int q0 = blockIdx.x * (NW * 32) + wave * 32;
-  int len = cu[b + 1] - cu[b];
-  len = len < 0 ? 0 : (len > seq ? seq : len);
+  const int cuLo = cu[b], cuHi = cu[b + 1]; // consumed after the first loads are out
 
   const int64_t tokStride = int64_t(3) * heads * kHeadDim;
   const _Float16 *base = qkv + int64_t(b) * seq * tokStride;
@@ -73,6 +72,46 @@ __global__ __launch_bounds__(NW *kWave) void bertAttentionKernel(
   const int64_t outStride = int64_t(heads) * kHeadDim;
   _Float16 *oBase = out + int64_t(b) * seq * outStride + head * kHeadDim;
 
+  // 2-wavefront variant (short sequences, few workgroups: latency is what
+  // counts): K and V rows of a 128-key chunk travel global -> registers -> LDS,
+  // 16 bytes per vector.  The loads are unconditional (rows past the end of the tensor
+  // are clamped, rows past the sequence end are zeroed on the way to LDS), so
+  // the first chunk's loads and the Q loads are issued before the sequence
+  // length has arrived, and the next chunk's loads fly while this one is
+  // multiplied.  The 4-wavefront variant serves long sequences with many
+  // workgroups per CU, which cover each other's staging; there the early loads
+  // are wasted on all-padding workgroups and the plain copy loop measured 3-8 %
+  // faster.
+  constexpr bool kPrefetch = NW == 2;
+  constexpr int VPT = kChunk * 8 / kThreads; // vectors of K (and of V) per thread
+  half8 rk[VPT], rv[VPT];
+  auto loadChunk = [&](int key0) {
+#pragma unroll
+    for (int i = 0; i < VPT; i++) {
+      const int v = tid + i * kThreads;
+      const int r = v / 8, c = v % 8;
+      const int row = key0 + r < seq ? key0 + r : seq - 1;
+      rk[i] = *reinterpret_cast<const half8 *>(kBase + int64_t(row) * tokStride + c * 8);
+      rv[i] = *reinterpret_cast<const half8 *>(vBase + int64_t(row) * tokStride + c * 8);
+    }
+  };
+  if (kPrefetch)
+    loadChunk(0);
+  // Q fragments (B operand of S^T = K Q^T): lane (q = l32, hb) holds
+  // Q[q][kk*16 + hb*8 .. +8] for kk = 0..3, pre-multiplied by nothing: the scale
+  // is applied to the fp32 scores.
+  half8 fq[kHeadDim / 16];
+  {
+    // rows past the tensor are clamped: what they produce is never stored
+    const int q = q0 + l32 < seq ? q0 + l32 : seq - 1;
+#pragma unroll
+    for (int kk = 0; kk < kHeadDim / 16; kk++)
+      fq[kk] = *reinterpret_cast<const half8 *>(qBase + int64_t(q) * tokStride +
+                                                kk * 16 + hb * 8);
+  }
+
+  int len = cuHi - cuLo;
+  len = len < 0 ? 0 : (len > seq ? seq : len);
   // A workgroup whose query rows are all padding has nothing to compute.
   if (int(blockIdx.x) * (NW * 32) >= len) {
     const int q = q0 + l32;
@@ -89,32 +128,14 @@ __global__ __launch_bounds__(NW *kWave) void bertAttentionKernel(
     return;
   }
 
-  // Q fragments (B operand of S^T = K Q^T): lane (q = l32, hb) holds
-  // Q[q][kk*16 + hb*8 .. +8] for kk = 0..3, pre-multiplied by nothing: the scale
-  // is applied to the fp32 scores.
-  half8 fq[kHeadDim / 16];
-  {
-    const int q = q0 + l32;
-#pragma unroll
-    for (int kk = 0; kk < kHeadDim / 16; kk++) {
-      half8 v;
-#pragma unroll
-      for (int e = 0; e < 8; e++)
-        v[e] = _Float16(0);
-      if (q < seq)
-        v = *reinterpret_cast<const half8 *>(qBase + int64_t(q) * tokStride +
-                                             kk * 16 + hb * 8);
-      fq[kk] = v;
-    }
-  }
-
   float16v accO[2]; // O^T: two 32-wide d blocks
 #pragma unroll
   for (int d = 0; d < 2; d++)
 #pragma unroll
     for (int e = 0; e < 16; e++)
       accO[d][e] = 0.f;
-  float rowMax = -INFINITY, rowSum = 0.f;
+  float rowMax = -INFINITY, rowSum = 0.f; // rowMax in raw (unscaled) score units
+  const float scaleLog2e = scale * 1.44269504088896340736f;
 
   // Per-lane constants of the fragment addresses.
   const int swzLane = (l32 >> 1) & 7;          // K: (row >> 1) & 7 for row = 32*x + l32
@@ -132,19 +153,39 @@ __global__ __launch_bounds__(NW *kWave) void bertAttentionKernel(
     // ---- stage K and V rows [key0, key0 + live): 8 vectors of 16 bytes per row.
     // Rows past the sequence end are zero-filled: masked scores ignore K, but a
     // masked probability (0) times a non-finite V would poison the output.
-    for (int v = tid; v < live * 8; v += kThreads) {
-      const int r = v / 8, c = v % 8;
-      half8 kv, vv;
+    if (kPrefetch) {
 #pragma unroll
-      for (int e = 0; e < 8; e++)
-        kv[e] = vv[e] = _Float16(0);
-      if (key0 + r < len) {
-        kv = *reinterpret_cast<const half8 *>(kBase + int64_t(key0 + r) * tokStride + c * 8);
-        vv = *reinterpret_cast<const half8 *>(vBase + int64_t(key0 + r) * tokStride + c * 8);
+      for (int i = 0; i < VPT; i++) {
+        const int v = tid + i * kThreads;
+        const int r = v / 8, c = v % 8;
+        if (r < live) {
+          half8 kv = rk[i], vv = rv[i];
+          if (key0 + r >= len) {
+#pragma unroll
+            for (int e = 0; e < 8; e++)
+              kv[e] = vv[e] = _Float16(0);
+          }
+          *reinterpret_cast<half8 *>(sK + r * 128 + swzK(r, c) * 16) = kv;
+          *reinterpret_cast<half8 *>(sV + r * 128 + swzV(r, c / 4) * 64 + (c % 4) * 16) = vv;
+        }
       }
-      *reinterpret_cast<half8 *>(sK + r * 128 + swzK(r, c) * 16) = kv;
-      *reinterpret_cast<half8 *>(sV + r * 128 + swzV(r, c / 4) * 64 + (c % 4) * 16) = vv;
+    } else {
+      for (int v = tid; v < live * 8; v += kThreads) {
+        const int r = v / 8, c = v % 8;
+        half8 kv, vv;
+#pragma unroll
+        for (int e = 0; e < 8; e++)
+          kv[e] = vv[e] = _Float16(0);
+        if (key0 + r < len) {
+          kv = *reinterpret_cast<const half8 *>(kBase + int64_t(key0 + r) * tokStride + c * 8);
+          vv = *reinterpret_cast<const half8 *>(vBase + int64_t(key0 + r) * tokStride + c * 8);
+        }
+        *reinterpret_cast<half8 *>(sK + r * 128 + swzK(r, c) * 16) = kv;
+        *reinterpret_cast<half8 *>(sV + r * 128 + swzV(r, c / 4) * 64 + (c % 4) * 16) = vv;
+      }
     }
+    if (kPrefetch && ch + 1 < numChunks)
+      loadChunk(key0 + kChunk);
     __syncthreads();
 
     for (int blk = 0; blk < live; blk += 64) {
@@ -163,29 +204,42 @@ __global__ __launch_bounds__(NW *kWave) void bertAttentionKernel(
                                                             0, 0, 0);
         }
       }
-      // accS[sb][e] is the score of query l32 against key
+      // accS[sb][e] is the raw score (before scaling) of query l32 against key
       //   key0 + blk + sb*32 + 8*(e/4) + 4*hb + e%4.
+      // The softmax works on raw scores: with c = scale * log2(e) > 0,
+      // exp(scale * (s - m)) = exp2(c * s - c * m), one FMA and one v_exp per
+      // score; the running maximum is kept in raw units.  Only a block that
+      // reaches past the sequence end pays for the key mask.  This part is
+      // VALU work the matrix core cannot hide (16 MFMAs against several
+      // hundred vector instructions per block), so instruction count matters.
+      if (key0 + blk + 64 > len) {
+#pragma unroll
+        for (int sb = 0; sb < 2; sb++)
+#pragma unroll
+          for (int e = 0; e < 16; e++) {
+            const int key = key0 + blk + sb * 32 + 8 * (e / 4) + 4 * hb + (e % 4);
+            accS[sb][e] = key < len ? accS[sb][e] : -INFINITY;
+          }
+      }
       float blockMax = -INFINITY;
 #pragma unroll
       for (int sb = 0; sb < 2; sb++)
 #pragma unroll
-        for (int e = 0; e < 16; e++) {
-          const int key = key0 + blk + sb * 32 + 8 * (e / 4) + 4 * hb + (e % 4);
-          const float s = key < len ? accS[sb][e] * scale : -INFINITY;
-          accS[sb][e] = s;
-          blockMax = fmaxf(blockMax, s);
-        }
+        for (int e = 0; e < 16; e++)
+          blockMax = fmaxf(blockMax, accS[sb][e]);
       blockMax = fmaxf(blockMax, __shfl_xor(blockMax, 32, kWave));
       const float newMax = fmaxf(rowMax, blockMax);
       // Every block that is visited has at least one valid key, so newMax is
       // finite and the differences below are never inf - inf.
-      const float corr = __expf(rowMax - newMax);
+      const float corr = __builtin_amdgcn_exp2f((rowMax - newMax) * scaleLog2e);
+      const float negMax = -newMax * scaleLog2e;
       float blockSum = 0.f;
 #pragma unroll
       for (int sb = 0; sb < 2; sb++)
 #pragma unroll
         for (int e = 0; e < 16; e++) {
-          const float pv = __expf(accS[sb][e] - newMax);
+          const float pv =
+              __builtin_amdgcn_exp2f(fmaf(accS[sb][e], scaleLog2e, negMax));
           accS[sb][e] = pv;
           blockSum += pv;
         }
@@ -264,6 +318,10 @@ Status launchBertAttentionF16(const _Float16 *qkv, const int32_t *cuSeqlens,
   HOM_CHECK_RET(headDim == kHeadDim, Status::kInvalidArgument,
                 "attention: head size %lld not supported (only 64)",
                 (long long)headDim);
+  // The softmax tracks the maximum of the unscaled scores, which is the
+  // maximum of the scaled ones only for a positive scale (BERT: 1/sqrt(64)).
+  HOM_CHECK_RET(scale > 0.f, Status::kInvalidArgument,
+                "attention: scale must be positive (got %g)", double(scale));
   HOM_CHECK_RET(bs < 65536 && heads < 65536 && seq < (int64_t(1) << 24),
                 Status::kInvalidArgument, "attention: shape out of range");
   HOM_CHECK_RET((reinterpret_cast<uintptr_t>(qkv) & 15) == 0 &&

@@ -43,6 +43,7 @@
 //    B is interleaved into (k, k+1) half2 pairs while it is staged.
 #include "kernels.h"
 
+#include <algorithm>
 #include <type_traits>
 #include <utility>
 
@@ -85,24 +86,25 @@ struct GemmParams {
   int kTilesPerSlice;
 };
 
-// GELU(x) = 0.5 x (1 + erf(x / sqrt 2)) with erfc(|z|) = t (a1 + t (a2 + ...))
-// exp(-z^2), t = 1 / (1 + p |z|) (Abramowitz & Stegun 7.1.26, |error| <=
-// 1.5e-7 on erfc, far below half a unit of the fp16 result):
-//   x >= 0: 1 + erf(z) = 2 - erfc(z);   x < 0: 1 + erf(z) = erfc(|z|)
-// so GELU(x) = max(x, 0) - 0.5 |x| erfc(|z|), with no cancellation on the
-// negative side.  A third of the instructions of the library erff.
+// GELU(x) = 0.5 x (1 + erf(x / sqrt 2)) = max(x, 0) - 0.5 |x| erfc(|x| / sqrt 2)
+// (x >= 0: 1 + erf = 2 - erfc; x < 0: 1 + erf = erfc(|z|); no cancellation on
+// the negative side), with erfc(a / sqrt 2) = 2^P(a): P is the degree-6 least
+// squares fit of log2 erfc(a / sqrt 2) on [0, 8], weighted by the sensitivity
+// of GELU to it.  Absolute error <= 2.7e-7 over fp32 inputs (the fp32 rounding
+// of the result itself near |x| = 4), at most one fp16 ulp away from the
+// exactly rounded value.  Beyond a = 8 the factor stays at 2^P(8) ~ 1e-15.
+// Six FMAs and one exp2: the epilogue runs when no MFMA work is left to hide
+// it, so its instruction count is wall time; the library erff costs 3x this.
 __device__ __forceinline__ float geluErf(float x) {
   const float ax = fabsf(x);
-  const float t =
-      __builtin_amdgcn_rcpf(fmaf(0.3275911f * 0.70710678118654752440f, ax, 1.0f));
-  float poly = fmaf(1.061405429f, t, -1.453152027f);
-  poly = fmaf(poly, t, 1.421413741f);
-  poly = fmaf(poly, t, -0.284496736f);
-  poly = fmaf(poly, t, 0.254829592f);
-  // exp(-x^2 / 2) = exp2(-x^2 * 0.5 * log2(e))
-  const float e = __builtin_amdgcn_exp2f(ax * ax * -0.72134752044448170368f);
-  const float erfcAbs = poly * t * e;
-  return fmaf(-0.5f * ax, erfcAbs, fmaxf(x, 0.0f));
+  const float a = fminf(ax, 8.0f);
+  float P = fmaf(3.448796997e-05f, a, -7.812886615e-04f);
+  P = fmaf(P, a, 8.119936101e-03f);
+  P = fmaf(P, a, -5.347220227e-02f);
+  P = fmaf(P, a, -4.587264359e-01f);
+  P = fmaf(P, a, -1.151216269e+00f);
+  P = fmaf(P, a, 8.451195754e-06f);
+  return fmaf(-0.5f * ax, __builtin_amdgcn_exp2f(P), fmaxf(x, 0.0f));
 }
 // 0.5 x (1 + tanh(u)) == x / (1 + exp(-2u)), u = sqrt(2/pi) (x + 0.044715 x^3)
 __device__ __forceinline__ float geluTanh(float x) {
@@ -121,8 +123,7 @@ template <int EPI> __device__ __forceinline__ float activate(float v) {
 }
 
 // XCD-contiguous tile id for this workgroup.
-__device__ __forceinline__ int tileForBlock(int nTiles) {
-  const int pid = blockIdx.x;
+__device__ __forceinline__ int tileForBlock(int nTiles, int pid) {
   const int q = nTiles / kNumXcd, r = nTiles % kNumXcd;
   const int xcd = pid % kNumXcd, loc = pid / kNumXcd;
   return xcd * q + (xcd < r ? xcd : r) + loc;
@@ -373,7 +374,7 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmDmaKernel(GemmParams p) {
   const int l32 = lane % 32, kb = lane / 32;
 
   const int nTiles = p.tilesM * p.tilesN;
-  const int tile = tileForBlock(nTiles);
+  const int tile = tileForBlock(nTiles, blockIdx.x);
   int tileM, tileN;
   tileCoords(tile, p.tilesM, p.tilesN, &tileM, &tileN);
   const int m0 = tileM * BM, n0 = tileN * BN;
@@ -616,8 +617,16 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(GemmParams p) {
   const int waveM = wave / WN, waveN = wave % WN;
   const int l32 = lane % 32, kb = lane / 32;
 
+  // Persistent over tiles: the grid holds at most as many workgroups as fit on
+  // the chip at once and each walks tiles pid, pid + grid, ...  (the grid is a
+  // multiple of the XCD count, so a workgroup's tiles stay in its XCD's
+  // contiguous range).  A tile's output stores drain and the next tile's first
+  // slabs arrive while other work runs, instead of between two workgroups.
   const int nTiles = p.tilesM * p.tilesN;
-  const int tile = tileForBlock(nTiles);
+  for (int vpid = blockIdx.x; vpid < nTiles; vpid += gridDim.x) {
+  if (vpid != int(blockIdx.x))
+    __syncthreads(); // the previous tile's epilogue strips live in this LDS
+  const int tile = tileForBlock(nTiles, vpid);
   int tileM, tileN;
   tileCoords(tile, p.tilesM, p.tilesN, &tileM, &tileN);
   const int m0 = tileM * BM, n0 = tileN * BN;
@@ -939,12 +948,13 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(GemmParams p) {
 
   if (numSlices > 1) {
     storePartial<MI, NI, THREADS>(p, acc, tile, slice, numSlices, tid);
-    return;
+    continue;
   }
   static_assert(WM * WN * 32 * (WTN * 4 + 16) <= 2 * STAGE_BYTES,
                 "epilogue strips must fit the main loop's LDS");
   epilogueStoreLds<MI, NI, WTM, WTN, EPI>(p, acc, m0, n0, waveM, waveN, lane,
                                           wave, smem);
+  } // tiles of this workgroup
 }
 
 // ================================================================== staged ==
@@ -971,7 +981,7 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmStagedKernel(GemmParams p) 
   const int waveM = wave / WN, waveN = wave % WN;
 
   const int nTiles = p.tilesM * p.tilesN;
-  const int tile = tileForBlock(nTiles);
+  const int tile = tileForBlock(nTiles, blockIdx.x);
   int tileM, tileN;
   tileCoords(tile, p.tilesM, p.tilesN, &tileM, &tileN);
   const int m0 = tileM * BM, n0 = tileN * BN;
@@ -1356,8 +1366,27 @@ Status launchPipe(const GemmProblem &pr, hipStream_t s) {
     return st;
   if (plan.nTiles == 0)
     return Status::kSuccess;
-  kernel<<<dim3((unsigned)plan.nTiles, (unsigned)plan.splitK),
-           dim3(WM * WN * kWave), SMEM, s>>>(plan.p);
+  // Workgroups that fit on the chip at once (rounded down to a multiple of the
+  // XCD count, which the tile order relies on); more tiles than that are walked
+  // by the same workgroups.
+  static int resident = 0;
+  if (resident == 0) {
+    int perCu = 0;
+    HOM_HIP_RET(hipOccupancyMaxActiveBlocksPerMultiprocessor(
+                    &perCu, kernel, WM * WN * kWave, SMEM),
+                Status::kInternal);
+    const int cus = deviceInfo().computeUnits > 0 ? deviceInfo().computeUnits : 256;
+    resident = perCu > 0 ? perCu * cus / kNumXcd * kNumXcd : 0;
+    if (resident < kNumXcd)
+      resident = 1 << 30; // unknown: one workgroup per tile
+  }
+  int64_t gridX = plan.nTiles;
+  if (gridX * plan.splitK > resident)
+    gridX = std::max<int64_t>(kNumXcd, resident / plan.splitK / kNumXcd * kNumXcd);
+  if (gridX > plan.nTiles)
+    gridX = plan.nTiles;
+  kernel<<<dim3((unsigned)gridX, (unsigned)plan.splitK), dim3(WM * WN * kWave),
+           SMEM, s>>>(plan.p);
   HOM_HIP_RET(hipGetLastError(), Status::kInternal);
   if (plan.splitK > 1)
     return launchReduce<BM, BN, WM, WN, EPI, 8>(plan, s);
