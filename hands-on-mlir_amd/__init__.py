@@ -14,6 +14,7 @@ CSRC_DIR = os.path.join(PKG_DIR, "csrc")
 LIB_DIR = os.path.join(PKG_DIR, "lib")
 RUNTIME_LIB = os.path.join(LIB_DIR, "libhom_amdgpu_runner_utils.so")
 DRIVER_LIB = os.path.join(LIB_DIR, "libhom_bert_driver.so")
+ENGINE_LIB = os.path.join(LIB_DIR, "libhom_execution_engine.so")
 
 
 def build(jobs: int = 8, force: bool = True) -> None:

@@ -755,13 +755,99 @@ C_UnrankedMemRefType allocDevice(const std::vector<int64_t> &sizes,
 
 // Text format written by the reference's weight serialiser
 // (lib/WeightsEngine/WeightsEngine.cpp:22-39) and read back by
-// allocConstantNVGPU* (HandsOnNVGPURunnerUtils.cu:224-298): first line the
-// three extents, then the values as decimal text.
+// Binary constant file "<idx>.bin": the 40-byte little-endian header below
+// (magic "HOMW", version 1, bytes per element: 2 = fp16 or 4 = fp32, rank 3, the
+// three extents), then the values, row-major.  Values of the constant's own
+// type are uploaded as they are; the other type is converted (fp32 -> fp16
+// rounds to nearest even, like the text path).
+struct ConstantHeader {
+  char magic[4];
+  uint32_t version;
+  uint32_t elementBytes;
+  uint32_t rank;
+  int64_t extents[3];
+};
+static_assert(sizeof(ConstantHeader) == 40, "constant file header layout");
+
+template <typename T>
+bool loadBinaryConstant(const std::string &path, int32_t idx,
+                        C_UnrankedMemRefType *res, bool *failed) {
+  FILE *f = fopen(path.c_str(), "rb");
+  if (!f)
+    return false; // no binary file: the caller falls back to the text format
+  *failed = true;
+  ConstantHeader h{};
+  const bool headOk = fread(&h, sizeof(h), 1, f) == 1 &&
+                      memcmp(h.magic, "HOMW", 4) == 0 && h.version == 1 &&
+                      h.rank == 3 && (h.elementBytes == 2 || h.elementBytes == 4);
+  if (!headOk) {
+    fclose(f);
+    recordError(__FILE__, __LINE__, "constant %d: %s is not a HOMW v1 rank-3 file",
+                idx, path.c_str());
+    return true;
+  }
+  const int64_t total = h.extents[0] * h.extents[1] * h.extents[2];
+  if (h.extents[0] < 0 || h.extents[1] < 0 || h.extents[2] < 0) {
+    fclose(f);
+    recordError(__FILE__, __LINE__, "constant %d: negative extent in %s", idx,
+                path.c_str());
+    return true;
+  }
+  std::vector<unsigned char> raw(size_t(total) * h.elementBytes);
+  const size_t got = total ? fread(raw.data(), h.elementBytes, size_t(total), f) : 0;
+  fclose(f);
+  if (int64_t(got) != total) {
+    recordError(__FILE__, __LINE__,
+                "constant %d: %s holds %lld values, expected %lld", idx,
+                path.c_str(), (long long)got, (long long)total);
+    return true;
+  }
+  std::vector<T> conv;
+  const void *src = raw.data();
+  if (h.elementBytes != sizeof(T)) {
+    conv.resize(size_t(total));
+    for (int64_t i = 0; i < total; i++) {
+      if (h.elementBytes == 4) {
+        float v;
+        memcpy(&v, raw.data() + size_t(i) * 4, 4);
+        conv[size_t(i)] = T(v);
+      } else {
+        _Float16 v;
+        memcpy(&v, raw.data() + size_t(i) * 2, 2);
+        conv[size_t(i)] = T(v);
+      }
+    }
+    src = conv.data();
+  }
+  *res = allocDevice({h.extents[0], h.extents[1], h.extents[2]}, sizeof(T));
+  if (!res->descriptor)
+    return true;
+  if (total > 0) {
+    hipError_t e = hipMemcpy(hom_memref_data(res->descriptor), src,
+                             size_t(total) * sizeof(T), hipMemcpyHostToDevice);
+    if (e != hipSuccess) {
+      recordError(__FILE__, __LINE__, "constant %d: upload failed: %s", idx,
+                  hipGetErrorString(e));
+      return true;
+    }
+  }
+  *failed = false;
+  return true;
+}
+
+// allocConstantNVGPU* (HandsOnNVGPURunnerUtils.cu:224-298): "<idx>.txt" holds
+// the three extents on the first line, then the values as decimal text.  A
+// "<idx>.bin" beside it (or instead of it) is preferred: parsing 110 M decimal
+// weights takes minutes, reading them takes milliseconds.
 template <typename T> C_UnrankedMemRefType allocConstant(int32_t idx) {
   C_UnrankedMemRefType res{3, nullptr};
   const char *dir = getenv("HOM_CONSTANT_DIR");
-  std::string path = std::string(dir ? dir : ".") + "/" + std::to_string(idx) +
-                     ".txt";
+  const std::string stem =
+      std::string(dir ? dir : ".") + "/" + std::to_string(idx);
+  bool failed = false;
+  if (loadBinaryConstant<T>(stem + ".bin", idx, &res, &failed))
+    return res;
+  std::string path = stem + ".txt";
   FILE *f = fopen(path.c_str(), "rb");
   HOM_CHECK_RET(f != nullptr, res, "constant %d: cannot open %s (%s)", idx,
                 path.c_str(), strerror(errno));

@@ -1,11 +1,13 @@
 """CPU-side checks of the drop-in boundary: the library loads, exports every
 symbol the header declares, and rejects bad arguments before touching the GPU."""
 import ctypes
+import importlib
 import os
 import re
 import subprocess
 import sys
 
+import numpy as np
 import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
@@ -169,3 +171,24 @@ def test_constant_loader_rejects_bad_files(rt, tmp_path, monkeypatch):
     assert "cannot open" in _errors(rt, lambda lib: lib.allocConstantNVGPUF16(99))
     assert "expected 3" in _errors(rt, lambda lib: lib.allocConstantNVGPUF16(1))
     assert "holds 5 values, expected 6" in _errors(rt, lambda lib: lib.allocConstantNVGPUF16(2))
+
+
+def test_binary_constant_files(rt, tmp_path, monkeypatch):
+    """Writer layout (40-byte header, raw values) and the loader's header checks."""
+    import struct
+    weights = importlib.import_module("hands-on-mlir_amd.weights")
+    a = (np.arange(24, dtype=np.float32) * 0.37 - 3).reshape(2, 3, 4).astype(np.float16)
+    path = weights.write_binary(str(tmp_path), 7, a)
+    raw = open(path, "rb").read()
+    assert len(raw) == 40 + 48
+    assert struct.unpack("<4sIIIqqq", raw[:40]) == (b"HOMW", 1, 2, 3, 2, 3, 4)
+    assert np.array_equal(np.frombuffer(raw[40:], np.float16).reshape(2, 3, 4), a)
+    text = open(weights.write_text(str(tmp_path), 8, a[0])).read().split("\n")
+    assert text[0] == "1 3 4"
+    assert np.array_equal(np.array(text[1].split(), np.float32).astype(np.float16), a[0].ravel())
+    monkeypatch.setenv("HOM_CONSTANT_DIR", str(tmp_path))
+    (tmp_path / "3.bin").write_bytes(b"NOPE" + raw[4:])
+    (tmp_path / "4.bin").write_bytes(raw[:-2])
+    assert "not a HOMW v1 rank-3 file" in _errors(rt, lambda lib: lib.allocConstantNVGPUF16(3))
+    assert "holds 23 values, expected 24" in _errors(rt, lambda lib: lib.allocConstantNVGPUF16(4))
+

@@ -6,6 +6,7 @@ Tolerances (written where they are used):
   elementwise, gather, cu_seqlens: bit exact.
 """
 import ctypes
+import importlib
 
 import numpy as np
 import pytest
@@ -360,3 +361,17 @@ def test_alloc_family_and_constant_loader(gpu, rt, tmp_path, monkeypatch):
         want = vals.astype(np.float16 if dt == torch.float16 else np.float32)
         assert np.array_equal(host(out), want)
         gpu.deallocNVGPUF16(m.rank, m.descriptor)
+    # binary files win over text ones; either element size feeds either entry point
+    weights = importlib.import_module("hands-on-mlir_amd.weights")
+    weights.write_binary(str(tmp_path), 5, (vals * 2).reshape(2, 3, 4).astype(np.float16))
+    weights.write_binary(str(tmp_path), 6, (vals * 3).reshape(2, 3, 4).astype(np.float32))
+    for idx, scale in ((5, 2), (6, 3)):
+        for fn, dt in [(gpu.allocConstantNVGPUF16, torch.float16), (gpu.allocConstantNVGPUF32, torch.float32)]:
+            m = fn(idx)
+            ptr, sizes, _ = rt.read_descriptor(m)
+            assert sizes == [2, 3, 4]
+            out = torch.empty(24, dtype=dt, device="cuda")
+            assert hip.hipMemcpy(out.data_ptr(), ptr, 24 * out.element_size(), 3) == 0
+            src = (vals * scale).astype(np.float16 if idx == 5 else np.float32)
+            assert np.array_equal(host(out), src.astype(np.float16 if dt == torch.float16 else np.float32))
+            gpu.deallocNVGPUF16(m.rank, m.descriptor)
