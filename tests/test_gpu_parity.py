@@ -186,6 +186,22 @@ def test_gemm_every_manifest_kernel(gpu, rt, oracle):
                 assert_close(got[0], want, **GEMM_TOL, what=f"{name} {M_}x{N_}x{K_} splitK={sk}")
 
 
+def test_gemm_more_tiles_than_resident_workgroups(gpu, rt, oracle):
+    """Ragged problem whose tile count exceeds what the chip holds at once, so the
+    persistent kernels walk several tiles per workgroup (with and without split-K)."""
+    g = np.random.default_rng(35)
+    M_, N_, K_ = 4100, 4104, 136
+    A = g.standard_normal((1, M_, K_)).astype(np.float16)
+    B = (g.standard_normal((1, K_, N_)) * 0.1).astype(np.float16)
+    bias = g.standard_normal((1, 1, N_)).astype(np.float16)
+    want = oracle.gemm(A[0], B[0], bias[0], beta=1.0, act="gelu_erf")
+    for tile in ("64x64_64x2r2_w2x2", "128x128_64x2r2_w2x4", "256x256_64x2r1_w2x4"):
+        for sk in (1, 2):
+            got = run_gemm(gpu, rt, A, B, bias, np.zeros((1, M_, N_), np.float16), knum(rt, tile, "gelu"), sk,
+                           beta=1.0)
+            assert_close(got[0], want, **GEMM_TOL, what=f"{tile} splitK={sk}, {M_}x{N_}x{K_}")
+
+
 def test_gemm_config1_bias_gelu(gpu, rt, oracle, synth):
     c = synth.gemm_bias_gelu()
     for form, act in (("gelu_tanh", 2), ("gelu_erf", 1)):
