@@ -147,7 +147,8 @@ def main():
                                         "dense_TFLOP/s": 402653184 / (at_ms * 1e-3) / 1e12}
     for (m, n, k, act, tag) in [(16384, 4096, 1024, 1, "gemm_gelu_16384x4096x1024"),
                                 (16384, 1024, 4096, 0, "gemm_16384x1024x4096"),
-                                (64, 1024, 4096, 0, "gemm_skinny_64x1024x4096")]:
+                                (64, 1024, 4096, 0, "gemm_skinny_64x1024x4096"),
+                                (1024, 30522, 768, 0, "gemm_vocab_1024x30522x768")]:
         lib.homGemmSelect(m, n, k, act, ctypes.byref(idx), ctypes.byref(sk))
         t = drv.homTimeGemm(m, n, k, act, 0, idx.value + 1, sk.value, 100 if m > 1024 else 1000, 10)
         tf = 2.0 * m * n * k / (t * 1e-3) / 1e12

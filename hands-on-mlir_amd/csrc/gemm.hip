@@ -62,6 +62,7 @@ template <int N, class F> __device__ __forceinline__ void staticFor(F &&f) {
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 typedef float float16v __attribute__((ext_vector_type(16)));
 typedef float float4v __attribute__((ext_vector_type(4)));
 typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
@@ -154,6 +155,8 @@ __device__ __forceinline__ void epilogueStore(const GemmParams &p,
                                               int lane) {
   const int l32 = lane % 32, kb = lane / 32;
   const bool useC = p.beta != 0.f;
+  // 8-byte accesses need rows of C and D that start 8-byte aligned
+  const bool quadRows = p.ldd % 4 == 0 && (!useC || p.ldc % 4 == 0);
 #pragma unroll
   for (int i = 0; i < MI; i++) {
     const int m = m0 + waveM * WTM + i * 32 + l32;
@@ -166,9 +169,7 @@ __device__ __forceinline__ void epilogueStore(const GemmParams &p,
 #pragma unroll
       for (int g = 0; g < 4; g++) {
         const int n = n0 + waveN * WTN + j * 32 + g * 8 + kb * 4;
-        if (VEC == 8) {
-          if (n >= p.N)
-            continue;
+        if (VEC == 8 && quadRows && n + 4 <= p.N) {
           float c[4] = {0.f, 0.f, 0.f, 0.f};
           if (useC) {
             const half4 cv = *reinterpret_cast<const half4 *>(p.C + cRow + n);
@@ -222,6 +223,8 @@ epilogueStoreLds(const GemmParams &p, float16v (&acc)[MI][NI], int m0, int n0,
   const bool useC = p.beta != 0.f;
   const int rr = lane / LPR, cc = (lane % LPR) * 8;
   const int n = n0 + waveN * WTN + cc;
+  // 16-byte accesses need rows of C and D that start 16-byte aligned
+  const bool vec16 = p.ldd % 8 == 0 && (!useC || p.ldc % 8 == 0);
   __syncthreads();
 #pragma unroll
   for (int i = 0; i < MI; i++) {
@@ -245,13 +248,26 @@ epilogueStoreLds(const GemmParams &p, float16v (&acc)[MI][NI], int m0, int n0,
           *reinterpret_cast<const float4v *>(mine + r * ROW_B + cc * 4 + 16);
       const int m = m0 + waveM * WTM + i * 32 + r;
       if (m < p.M && n < p.N) {
+        const _Float16 *cPtr = p.C + int64_t(m % p.cRowPeriod) * p.ldc + n;
+        _Float16 *dPtr = p.D + int64_t(m) * p.ldd + n;
         float c[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
         if (useC) {
-          const half8 cv = *reinterpret_cast<const half8 *>(
-              p.C + int64_t(m % p.cRowPeriod) * p.ldc + n);
+          if (vec16) {
+            const half8 cv = *reinterpret_cast<const half8 *>(cPtr);
 #pragma unroll
-          for (int e = 0; e < 8; e++)
-            c[e] = float(cv[e]);
+            for (int e = 0; e < 8; e++)
+              c[e] = float(cv[e]);
+          } else {
+            // rows start at 4-byte boundaries only (N not a multiple of 8):
+            // pairs, and the pair that reaches past column N is dropped (N even)
+#pragma unroll
+            for (int e = 0; e < 8; e += 2)
+              if (n + e < p.N) {
+                const half2v cv = *reinterpret_cast<const half2v *>(cPtr + e);
+                c[e] = float(cv[0]);
+                c[e + 1] = float(cv[1]);
+              }
+          }
         }
         half8 o;
 #pragma unroll
@@ -261,7 +277,18 @@ epilogueStoreLds(const GemmParams &p, float16v (&acc)[MI][NI], int m0, int n0,
             v += p.beta * c[e];
           o[e] = _Float16(activate<EPI>(v));
         }
-        *reinterpret_cast<half8 *>(p.D + int64_t(m) * p.ldd + n) = o;
+        if (vec16) {
+          *reinterpret_cast<half8 *>(dPtr) = o;
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; e += 2)
+            if (n + e < p.N) {
+              half2v ov;
+              ov[0] = o[e];
+              ov[1] = o[e + 1];
+              *reinterpret_cast<half2v *>(dPtr + e) = ov;
+            }
+        }
       }
     }
   }
@@ -1409,7 +1436,7 @@ struct KernelEntry {
   {                                                                            \
     {"hom_gfx950_mfma_f16_s32x32x16gemm_f16_" #BM "x" #BN "_64x" #NS "_w" #WM  \
      "x" #WN "_nn_align8_" EPI_STR,                                            \
-     BM, BN, 64, WM, WN, 8, ACT, EPI_ENUM},                                    \
+     BM, BN, 64, WM, WN, 8, 8, ACT, EPI_ENUM},                                 \
         launchDma<BM, BN, WM, WN, NS, int(EPI_ENUM), false>,                   \
         launchDma<BM, BN, WM, WN, NS, int(EPI_ENUM), true>                     \
   }
@@ -1424,7 +1451,7 @@ struct KernelEntry {
   {                                                                            \
     {"hom_gfx950_mfma_f16_s32x32x16gemm_f16_" #BM "x" #BN "_64x2r" #DIST FBS   \
      "_w" #WM "x" #WN "_nn_align8_" EPI_STR,                                   \
-     BM, BN, 64, WM, WN, 8, ACT, EPI_ENUM},                                    \
+     BM, BN, 64, WM, WN, 8, 2, ACT, EPI_ENUM},                                 \
         launchPipe<BM, BN, WM, WN, DIST, FB, int(EPI_ENUM), false>,            \
         launchPipe<BM, BN, WM, WN, DIST, FB, int(EPI_ENUM), true>              \
   }
@@ -1444,7 +1471,7 @@ struct KernelEntry {
   {                                                                            \
     {"hom_gfx950_mfma_f16_s32x32x16gemm_f16_" #BM "x" #BN "_" #BK "x2_w" #WM   \
      "x" #WN "_nn_align" #VEC "_" EPI_STR,                                     \
-     BM, BN, BK, WM, WN, VEC, ACT, EPI_ENUM},                                  \
+     BM, BN, BK, WM, WN, VEC, VEC, ACT, EPI_ENUM},                             \
         launchStaged<BM, BN, BK, WM, WN, int(EPI_ENUM), false, VEC>,           \
         launchStaged<BM, BN, BK, WM, WN, int(EPI_ENUM), true, VEC>             \
   }
@@ -1509,16 +1536,24 @@ Status launchGemm(int idx, const GemmProblem &p, hipStream_t s) {
                 "gemm: beta != 0 needs a source tensor");
   if (k.info.alignment == 8) {
     // What CUTLASS's can_implement() rejects: misaligned leading dimensions.
-    const bool ok = p.N % 8 == 0 && p.K % 8 == 0 && p.lda % 8 == 0 &&
-                    p.ldb % 8 == 0 && p.ldd % 8 == 0 &&
-                    (p.beta == 0.f || p.ldc % 8 == 0) && aligned16(p.A) &&
-                    aligned16(p.B) && aligned16(p.D) &&
-                    (p.beta == 0.f || aligned16(p.C));
+    // K-contiguous operands (A, and B given as [N, K]) are read 16 bytes at a
+    // time from 16-byte aligned rows; row-major B, C and D follow alignmentN.
+    const int an = k.info.alignmentN;
+    auto alignedTo = [](const void *q, int bytes) {
+      return (reinterpret_cast<uintptr_t>(q) & uintptr_t(bytes - 1)) == 0;
+    };
+    const bool ok =
+        p.K % 8 == 0 && p.lda % 8 == 0 && aligned16(p.A) && p.N % an == 0 &&
+        (p.bIsNK ? (p.ldb % 8 == 0 && aligned16(p.B))
+                 : (p.ldb % an == 0 && alignedTo(p.B, 2 * an))) &&
+        p.ldd % an == 0 && alignedTo(p.D, 2 * an) &&
+        (p.beta == 0.f || (p.ldc % an == 0 && alignedTo(p.C, 2 * an)));
     HOM_CHECK_RET(ok, Status::kInvalidArgument,
-                  "gemm: kernel %s needs N, K and leading dimensions that are "
-                  "multiples of 8 and 16-byte aligned operands (M=%lld N=%lld "
-                  "K=%lld)",
-                  k.info.name, (long long)p.M, (long long)p.N, (long long)p.K);
+                  "gemm: kernel %s needs K a multiple of 8, N and the leading "
+                  "dimensions of B, C, D multiples of %d, and operands aligned "
+                  "to match (M=%lld N=%lld K=%lld)",
+                  k.info.name, an, (long long)p.M, (long long)p.N,
+                  (long long)p.K);
   }
   if (p.M == 0 || p.N == 0)
     return Status::kSuccess;

@@ -82,7 +82,12 @@ struct GemmKernelInfo {
   const char *name;
   int tileM, tileN, tileK;
   int wavesM, wavesN;
-  int alignment; // required divisor of N and K (8 or 1)
+  int alignment; // required divisor of K (8: vector accesses, 1: any shape)
+  // Required divisor of N and of the leading dimensions of B (row-major), C, D
+  // (8, 2 or 1).  2: rows of B / C / D start at any 4-byte boundary, e.g. the
+  // 30522-wide vocabulary projection; the reference's manifest carries separate
+  // alignment 8/4/2/1 kernels for this (python/gemm_generator.py:237-278).
+  int alignmentN;
   int activation; // 0 linear, 1 gelu (what the profiler filters on)
   Epilogue epilogue;
 };

@@ -136,13 +136,44 @@ const TunedEntry kTuned[] = {
 #include "gemm_tuned_table.inc"
     {0, 0, 0, 0, nullptr, 0}};
 
+// 8: every operand 16-byte aligned with N, K multiples of 8; 2: K a multiple
+// of 8 and the K-contiguous operands 16-byte aligned, but N (the row length of
+// row-major B, C, D) only even; 1: anything else.
 int alignmentClass(const GemmProblem &p) {
-  auto a16 = [](const void *q) {
-    return (reinterpret_cast<uintptr_t>(q) & 15) == 0;
+  auto al = [](const void *q, int bytes) {
+    return (reinterpret_cast<uintptr_t>(q) & uintptr_t(bytes - 1)) == 0;
   };
-  const bool ok = p.N % 8 == 0 && p.K % 8 == 0 && a16(p.A) && a16(p.B) &&
-                  a16(p.D) && (p.C == nullptr || a16(p.C));
-  return ok ? 8 : 1;
+  if (p.K % 8 != 0 || !al(p.A, 16))
+    return 1;
+  const bool c8 = p.N % 8 == 0 && al(p.B, 16) && al(p.D, 16) &&
+                  (p.C == nullptr || al(p.C, 16));
+  if (c8)
+    return 8;
+  const bool c2 = p.N % 2 == 0 && (p.bIsNK ? al(p.B, 16) : al(p.B, 4)) &&
+                  al(p.D, 4) && (p.C == nullptr || al(p.C, 4)) &&
+                  (p.C == nullptr || p.ldc % 2 == 0);
+  return c2 ? 2 : 1;
+}
+
+// A vector-access kernel (alignment 8) serves the problem when the problem's
+// class is 8, or 2 and the kernel tolerates 4-byte aligned rows.
+bool kernelFits(const GemmKernelInfo &k, int cls) {
+  if (k.alignment == 1)
+    return true;
+  return cls == 8 || (cls == 2 && k.alignmentN <= 2);
+}
+
+// What to run when the selected kernel does not fit the problem's alignment.
+int fallbackKernel(Epilogue epi, int cls) {
+  if (cls == 2) {
+    for (int i = 0; i < gemmKernelCount(); i++) {
+      const GemmKernelInfo &k = gemmKernelInfo(i);
+      if (k.epilogue == epi && k.alignment == 8 && k.alignmentN <= 2 &&
+          k.tileM == 128 && k.tileN == 128)
+        return i;
+    }
+  }
+  return findKernel(64, 64, 32, epi, 1);
 }
 
 } // namespace
@@ -166,13 +197,14 @@ bool selectGemm(int64_t M, int64_t N, int64_t K, int64_t activation,
   // Heuristic: estimate each tile's time as (rounds of workgroups over the
   // chip) x (tile work / tile efficiency) and take the cheapest; small output
   // grids get split-K until the chip is covered.
-  const int align = (N % 8 == 0 && K % 8 == 0) ? 8 : 1;
+  const int cls = K % 8 != 0 ? 1 : (N % 8 == 0 ? 8 : (N % 2 == 0 ? 2 : 1));
   const int cus = deviceInfo().computeUnits > 0 ? deviceInfo().computeUnits : 256;
   double bestCost = 1e300;
   int best = -1, bestSplit = 1;
   for (int i = 0; i < gemmKernelCount(); i++) {
     const GemmKernelInfo &k = gemmKernelInfo(i);
-    if (k.epilogue != epi || k.alignment != align)
+    if (k.epilogue != epi || (cls == 1) != (k.alignment == 1) ||
+        !kernelFits(k, cls))
       continue;
     const int64_t tiles = ((M + k.tileM - 1) / k.tileM) *
                           ((N + k.tileN - 1) / k.tileN);
@@ -237,8 +269,9 @@ Status runGemmManifest(int64_t rankA, void *dstA, int64_t rankB, void *dstB,
     selectGemm(pr.M, pr.N, pr.K, activation, &sel, &sk);
     idx = int(sel);
     pr.splitK = sk;
-    if (gemmKernelInfo(idx).alignment == 8 && alignmentClass(pr) != 8) {
-      idx = findKernel(64, 64, 32, gemmKernelInfo(idx).epilogue, 1);
+    const int cls = alignmentClass(pr);
+    if (!kernelFits(gemmKernelInfo(idx), cls)) {
+      idx = fallbackKernel(gemmKernelInfo(idx).epilogue, cls);
       pr.splitK = 1;
     }
   }
@@ -293,8 +326,9 @@ Status runGemmNvte(int64_t rankA, void *dstA, bool transa, int64_t rankB,
         pr.splitK = comma == std::string::npos ? 1 : atoi(f.c_str() + comma + 1);
       }
   }
-  if (gemmKernelInfo(idx).alignment == 8 && alignmentClass(pr) != 8) {
-    idx = findKernel(64, 64, 32, epi, 1);
+  const int cls = alignmentClass(pr);
+  if (!kernelFits(gemmKernelInfo(idx), cls)) {
+    idx = fallbackKernel(epi, cls);
     pr.splitK = 1;
   }
   return launchGemm(idx, pr, stream());
@@ -461,10 +495,10 @@ std::tuple<int64_t, int32_t> GemmProfiler::profile() {
   if (!ensure(a_, M_ * K_) || !ensure(b_, K_ * N_) || !ensure(c_, M_ * N_))
     return {-1, 1};
   const Epilogue epi = epilogueFor(activation_, false);
-  // Alignment class: largest of {8, 1} dividing N and K (the reference walks
-  // {8,4,2,1} over M, N, K: lib/NVGPUKernels/GemmProfiler.cu:170-180; row
-  // count does not constrain these kernels).
-  const int align = (N_ % 8 == 0 && K_ % 8 == 0) ? 8 : 1;
+  // Alignment class (the reference walks {8,4,2,1} over M, N, K:
+  // lib/NVGPUKernels/GemmProfiler.cu:170-180; here K must be a multiple of 8
+  // for the vector kernels, N of 8 or 2, and the row count is free).
+  const int cls = K_ % 8 != 0 ? 1 : (N_ % 8 == 0 ? 8 : (N_ % 2 == 0 ? 2 : 1));
   const int maxSplit = std::max(1, std::min<int>(16, int(K_ / 128)));
   const int cus = deviceInfo().computeUnits > 0 ? deviceInfo().computeUnits : 256;
 
@@ -473,9 +507,9 @@ std::tuple<int64_t, int32_t> GemmProfiler::profile() {
   float bestTime = INFINITY;
   for (int idx = 0; idx < gemmKernelCount(); idx++) {
     const GemmKernelInfo &k = gemmKernelInfo(idx);
-    if (k.epilogue != epi || k.alignment > align)
+    if (k.epilogue != epi || !kernelFits(k, cls))
       continue;
-    if (k.alignment < align && align == 8)
+    if (k.alignment == 1 && cls != 1)
       continue; // the scalar-access kernels never win on aligned problems
     const int64_t tiles = ((M_ + k.tileM - 1) / k.tileM) *
                           ((N_ + k.tileN - 1) / k.tileN);

@@ -74,14 +74,18 @@ def test_select_returns_compatible_kernel(rt):
     man = rt.manifest()
     idx, sk = ctypes.c_int64(), ctypes.c_int32()
     for (M, N, K, act) in [(1024, 2304, 768, 0), (1024, 3072, 768, 1), (1024, 3072, 768, 2),
-                           (1024, 768, 3072, 0), (64, 1024, 4096, 0), (7, 13, 5, 0), (16384, 4096, 1024, 1)]:
+                           (1024, 768, 3072, 0), (64, 1024, 4096, 0), (7, 13, 5, 0), (16384, 4096, 1024, 1),
+                           (1024, 30522, 768, 0), (64, 250, 72, 1), (64, 251, 72, 0), (64, 256, 76, 0)]:
         lib.homGemmSelect(M, N, K, act, ctypes.byref(idx), ctypes.byref(sk))
         _, name, a, align = man[idx.value]
         assert a == (1 if act else 0)
         assert ("gelutanh" in name) == (act == 2)
         assert sk.value >= 1 and sk.value <= max(1, min(16, K // 128))
-        if N % 8 or K % 8:
+        if N % 2 or K % 8:
             assert align == 1
+        elif N % 8:
+            # even N: only the register-staged family reads rows that start at 4-byte boundaries
+            assert align == 8 and "_64x2r" in name
 
 
 # ---- argument checking: runs without a GPU because every check precedes the

@@ -202,6 +202,43 @@ def test_gemm_more_tiles_than_resident_workgroups(gpu, rt, oracle):
             assert_close(got[0], want, **GEMM_TOL, what=f"{tile} splitK={sk}, {M_}x{N_}x{K_}")
 
 
+def test_gemm_even_n_not_multiple_of_8(gpu, rt, oracle):
+    """N % 8 != 0 with K % 8 == 0: rows of B, C, D start at 4-byte boundaries only.
+    The register-staged kernels take these directly (the reference's alignment-2
+    CUTLASS instances); covers the BERT vocabulary projection width 30522."""
+    g = np.random.default_rng(36)
+    for (M_, N_, K_) in [(200, 250, 136), (64, 30522, 64), (130, 6, 72), (96, 1026, 768)]:
+        A = g.standard_normal((1, M_, K_)).astype(np.float16)
+        B = (g.standard_normal((1, K_, N_)) * 0.1).astype(np.float16)
+        bias = g.standard_normal((1, 1, N_)).astype(np.float16)
+        R = g.standard_normal((1, M_, N_)).astype(np.float16)
+        want_bias = oracle.gemm(A[0], B[0], bias[0], beta=1.0, act="gelu_erf")
+        want_res = oracle.gemm(A[0], B[0], R[0], beta=1.0)
+        for tile in ("64x64_64x2r2_w2x2", "128x128_64x2r2_w2x4", "256x256_64x2r1_w2x4"):
+            for sk in (1, 2):
+                got = run_gemm(gpu, rt, A, B, bias, np.zeros((1, M_, N_), np.float16), knum(rt, tile, "gelu"),
+                               sk, beta=1.0)
+                assert_close(got[0], want_bias, **GEMM_TOL, what=f"{tile} splitK={sk} {M_}x{N_}x{K_} bias+gelu")
+                got = run_gemm(gpu, rt, A, B, None, R, knum(rt, tile), sk, beta=1.0, in_place=True)
+                assert_close(got[0], want_res, **GEMM_TOL, what=f"{tile} splitK={sk} {M_}x{N_}x{K_} residual")
+        # the library's own choice (gemmNum 0) must not fall back to the scalar kernel
+        idx, sk = ctypes.c_int64(), ctypes.c_int32()
+        gpu.homGemmSelect(M_, N_, K_, 0, ctypes.byref(idx), ctypes.byref(sk))
+        name = rt.manifest()[idx.value][1]
+        assert "align8" in name and "r" in name.split("_64x2")[1][:2], name
+        got = run_gemm(gpu, rt, A, B, None, R, 0, 1, beta=1.0, in_place=True)
+        assert_close(got[0], want_res, **GEMM_TOL, what=f"auto {M_}x{N_}x{K_}")
+    # a kernel of the DMA family still refuses such a problem
+    A = g.standard_normal((1, 64, 64)).astype(np.float16)
+    B = g.standard_normal((1, 64, 250)).astype(np.float16)
+    gpu.homSetErrorMode(1)
+    try:
+        run_gemm(gpu, rt, A, B, None, np.zeros((1, 64, 250), np.float16), knum(rt, "128x128_64x4"), 1)
+        assert b"multiples of 8" in gpu.homGetLastError()
+    finally:
+        gpu.homSetErrorMode(0)
+
+
 def test_gemm_config1_bias_gelu(gpu, rt, oracle, synth):
     c = synth.gemm_bias_gelu()
     for form, act in (("gelu_tanh", 2), ("gelu_erf", 1)):
