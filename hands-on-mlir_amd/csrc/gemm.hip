@@ -621,9 +621,9 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmDmaKernel(GemmParams p) {
 // The vector memory path into registers sustains several times the bandwidth
 // of the LDS-DMA path on this chip, which matters once a CU streams more than
 // ~16 bytes per clock (large tiles, or several workgroups per CU).
-template <int BM, int BN, int WM, int WN, int DIST, int FB, int EPI, bool B_NK>
+template <int BM, int BN, int WM, int WN, int DIST, int EPI, bool B_NK>
 __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(GemmParams p) {
-  static_assert(DIST >= 1 && (FB == 1 || FB == 2), "unsupported pipeline shape");
+  static_assert(DIST >= 1, "at least one slab of global loads in flight");
   constexpr int BK = 64;
   constexpr int THREADS = WM * WN * kWave;
   constexpr int WTM = BM / WM, WTN = BN / WN;
@@ -828,14 +828,12 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(GemmParams p) {
   // register-set index a compile-time constant.
   // The barrier is a bare s_barrier behind an LDS-only wait: a fence here would
   // drain the global loads that were just issued.
-  // FB == 2 fetches the fragments of k step kk+1 before the MFMAs of step kk
-  // (two fragment sets); FB == 1 keeps one set and relies on the other
-  // wavefronts of the SIMD to cover the LDS latency, which frees registers for a
-  // deeper global pipeline on the largest tiles.
+  // The fragments of k step kk+1 are fetched under the MFMAs of step kk (two
+  // fragment sets).
   constexpr int NV = A_PER_T + B_PER_T; // vectors per thread and slab
   constexpr int NM = MI * NI;           // MFMAs per wavefront and k step
   constexpr int ST_STEPS = KSTEPS - 1;  // k steps that carry staging work
-  half8 fa[FB][MI], fb[FB][NI];
+  half8 fa[2][MI], fb[2][NI];
   const int nk = ktEnd - ktBegin;
   // Moves vector v of register set S to LDS and refills it from slab kt.
   auto stageVec = [&](int stage, int kt, auto setC, auto vC) {
@@ -910,40 +908,22 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(GemmParams p) {
       constexpr int V1 = kk < ST_STEPS ? (kk + 1) * NV / ST_STEPS : NV;
       using V0C = std::integral_constant<int, V0>;
       using V1C = std::integral_constant<int, V1>;
-      constexpr int cs = kk % FB, ns = (kk + 1) % FB;
+      constexpr int cs = kk % 2, ns = (kk + 1) % 2;
       if constexpr (kk < KSTEPS - 1) {
-        if constexpr (FB == 2) {
-          mfmaMixed(fa[cs], fb[cs], fa[ns], fb[ns], cur, kk + 1,
-                    std::true_type{}, cur ^ 1, ktNext, more, setC, V0C{},
-                    V1C{});
-        } else {
-          if (kk > 0)
-            loadFrags(cur, kk, fa[0], fb[0]);
-          __builtin_amdgcn_sched_barrier(0);
-          mfmaMixed(fa[0], fb[0], fa[0], fb[0], 0, 0, std::false_type{},
-                    cur ^ 1, ktNext, more, setC, V0C{}, V1C{});
-        }
+        mfmaMixed(fa[cs], fb[cs], fa[ns], fb[ns], cur, kk + 1, std::true_type{},
+                  cur ^ 1, ktNext, more, setC, V0C{}, V1C{});
       } else {
-        if constexpr (FB == 1) {
-          loadFrags(cur, kk, fa[0], fb[0]);
-          mfmaMixed(fa[0], fb[0], fa[0], fb[0], 0, 0, std::false_type{}, 0, 0,
-                    false, setC, V0C{}, V1C{});
-        }
+        static_assert(ns == 0, "the next slab finds its first fragments in set 0");
         if (more) {
           // Every wavefront has its last fragments of slab i in registers and
-          // slab i+1 is complete in the other buffer after this barrier.
+          // slab i+1 is complete in the other buffer after this barrier; its
+          // first fragments arrive under the MFMAs of the last k step.
           asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-        }
-        if constexpr (FB == 2) {
-          // ns == 0: the first fragments of slab i+1 arrive under these MFMAs
-          if (more)
-            mfmaMixed(fa[cs], fb[cs], fa[ns], fb[ns], cur ^ 1, 0,
-                      std::true_type{}, 0, 0, false, setC, V0C{}, V1C{});
-          else
-            mfmaMixed(fa[cs], fb[cs], fa[ns], fb[ns], 0, 0, std::false_type{},
-                      0, 0, false, setC, V0C{}, V1C{});
-        } else if (more) {
-          loadFrags(cur ^ 1, 0, fa[0], fb[0]);
+          mfmaMixed(fa[cs], fb[cs], fa[ns], fb[ns], cur ^ 1, 0, std::true_type{},
+                    0, 0, false, setC, V0C{}, V1C{});
+        } else {
+          mfmaMixed(fa[cs], fb[cs], fa[ns], fb[ns], 0, 0, std::false_type{}, 0,
+                    0, false, setC, V0C{}, V1C{});
         }
       }
     });
@@ -1372,7 +1352,7 @@ Status launchDma(const GemmProblem &pr, hipStream_t s) {
   return Status::kSuccess;
 }
 
-template <int BM, int BN, int WM, int WN, int DIST, int FB, int EPI, bool B_NK>
+template <int BM, int BN, int WM, int WN, int DIST, int EPI, bool B_NK>
 Status launchPipe(const GemmProblem &pr, hipStream_t s) {
   constexpr int SMEM = 2 * (BM + BN) * 64 * 2;
   LaunchPlan plan;
@@ -1386,7 +1366,7 @@ Status launchPipe(const GemmProblem &pr, hipStream_t s) {
   HOM_CHECK_RET((int64_t(BM) * pr.lda + pr.K) * 2 < (int64_t(1) << 31) &&
                     (int64_t(BN) * pr.ldb + pr.K) * 2 < (int64_t(1) << 31),
                 Status::kInvalidArgument, "gemm: leading dimension too large");
-  auto kernel = gemmPipeKernel<BM, BN, WM, WN, DIST, FB, EPI, B_NK>;
+  auto kernel = gemmPipeKernel<BM, BN, WM, WN, DIST, EPI, B_NK>;
   static bool attrSet = false;
   st = allowLds(kernel, SMEM, &attrSet);
   if (st != Status::kSuccess)
@@ -1446,26 +1426,19 @@ struct KernelEntry {
       HOM_DMA_ENTRY(BM, BN, WM, WN, NS, Epilogue::kGeluTanh, "gelutanh", 1)
 
 // "r<d>" after the LDS stage count marks the register-staged pipeline with d
-// slabs of global loads in flight; a trailing "s" a single fragment set.
-#define HOM_PIPE_ENTRY(BM, BN, WM, WN, DIST, FB, FBS, EPI_ENUM, EPI_STR, ACT)  \
+// slabs of global loads in flight.
+#define HOM_PIPE_ENTRY(BM, BN, WM, WN, DIST, EPI_ENUM, EPI_STR, ACT)           \
   {                                                                            \
-    {"hom_gfx950_mfma_f16_s32x32x16gemm_f16_" #BM "x" #BN "_64x2r" #DIST FBS   \
+    {"hom_gfx950_mfma_f16_s32x32x16gemm_f16_" #BM "x" #BN "_64x2r" #DIST       \
      "_w" #WM "x" #WN "_nn_align8_" EPI_STR,                                   \
      BM, BN, 64, WM, WN, 8, 2, ACT, EPI_ENUM},                                 \
-        launchPipe<BM, BN, WM, WN, DIST, FB, int(EPI_ENUM), false>,            \
-        launchPipe<BM, BN, WM, WN, DIST, FB, int(EPI_ENUM), true>              \
+        launchPipe<BM, BN, WM, WN, DIST, int(EPI_ENUM), false>,                \
+        launchPipe<BM, BN, WM, WN, DIST, int(EPI_ENUM), true>                  \
   }
-#define HOM_PIPE_TILE_FB(BM, BN, WM, WN, DIST, FB, FBS)                        \
-  HOM_PIPE_ENTRY(BM, BN, WM, WN, DIST, FB, FBS, Epilogue::kLinear, "linear",   \
-                 0),                                                           \
-      HOM_PIPE_ENTRY(BM, BN, WM, WN, DIST, FB, FBS, Epilogue::kGeluErf,        \
-                     "gelu", 1),                                               \
-      HOM_PIPE_ENTRY(BM, BN, WM, WN, DIST, FB, FBS, Epilogue::kGeluTanh,       \
-                     "gelutanh", 1)
 #define HOM_PIPE_TILE(BM, BN, WM, WN, DIST)                                    \
-  HOM_PIPE_TILE_FB(BM, BN, WM, WN, DIST, 2, "")
-#define HOM_PIPE_TILE_S(BM, BN, WM, WN, DIST)                                  \
-  HOM_PIPE_TILE_FB(BM, BN, WM, WN, DIST, 1, "s")
+  HOM_PIPE_ENTRY(BM, BN, WM, WN, DIST, Epilogue::kLinear, "linear", 0),        \
+      HOM_PIPE_ENTRY(BM, BN, WM, WN, DIST, Epilogue::kGeluErf, "gelu", 1),     \
+      HOM_PIPE_ENTRY(BM, BN, WM, WN, DIST, Epilogue::kGeluTanh, "gelutanh", 1)
 
 #define HOM_STAGED_ENTRY(BM, BN, BK, WM, WN, EPI_ENUM, EPI_STR, ACT, VEC)      \
   {                                                                            \
@@ -1489,7 +1462,6 @@ const KernelEntry kKernels[] = {
     HOM_DMA_TILE(64, 64, 2, 2, 4),
     HOM_DMA_TILE(128, 64, 2, 2, 4),
     HOM_DMA_TILE(64, 64, 2, 2, 8),
-    HOM_DMA_TILE(256, 256, 2, 4, 2),
     HOM_PIPE_TILE(64, 64, 2, 2, 2),
     HOM_PIPE_TILE(64, 64, 2, 2, 4),
     HOM_PIPE_TILE(128, 64, 2, 2, 2),
