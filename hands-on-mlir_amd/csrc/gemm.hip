@@ -669,11 +669,16 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(GemmParams p) {
   // row or column block (B): a constant 32-bit byte offset per thread plus a
   // scalar offset per slab.  Rows / columns past the edge are clamped to the
   // last valid one: what they fetch only reaches outputs that are never
-  // stored.  Vectors at or past kEnd (the K tail, and whole slabs requested
-  // beyond this slice) get an offset outside the descriptor and read as zero
-  // without touching memory, so every slab issues the same number of loads
-  // and the compiler's outstanding-load counts are exact -- a branch around a
-  // load makes it wait for everything in flight and defeats the pipeline.
+  // stored.  Every slab issues the same number of loads and there is no branch
+  // around a load, so the compiler's outstanding-load counts are exact (a
+  // branch makes it wait for everything in flight and defeats the pipeline).
+  // The main loop walks the slice's FULL slabs only and asks for no range
+  // test per vector: vector instructions in that loop cost matrix-core time.
+  // A slab requested past the last full one is replaced by the last full one
+  // (it is never used), and a partial last slab (K not a multiple of 64) is
+  // multiplied ahead of the loop by a short unpipelined pass whose loads map
+  // vectors at or past kEnd to an offset outside the descriptor (they read as
+  // zero without touching memory).
   constexpr uint32_t kOob = 0x80000000u;
   auto clampBytes = [](int64_t b) -> int32_t {
     return b > 0x7fffffffLL ? 0x7fffffff : (b < 0 ? 0 : int32_t(b));
@@ -690,7 +695,14 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(GemmParams p) {
       0x00020000);
   const int kEnd = ktEnd * BK < p.K ? ktEnd * BK : p.K;
   uint32_t aOff[A_PER_T], bOff[B_PER_T];
-  int aDst[A_PER_T], bDst[B_PER_T];
+  // LDS destination of vector i = destination of vector 0 + i * DST_STEP: the
+  // row advances by a multiple of 16 per vector, which leaves both swizzles
+  // unchanged (they depend on row bits 0..3 only).
+  constexpr int DST_STEP = THREADS * 16;
+  static_assert((THREADS / 8) % 16 == 0 && (THREADS / B_VPR) % 4 == 0 &&
+                    (BN != 64 || (THREADS / B_VPR) % 4 == 0),
+                "vector step must preserve the LDS swizzles");
+  int aDst0 = 0, bDst0 = 0;
   int aK[A_PER_T], bK[B_PER_T]; // k position inside the slab
 #pragma unroll
   for (int i = 0; i < A_PER_T; i++) {
@@ -699,7 +711,8 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(GemmParams p) {
     const int rr = m0 + r < p.M ? r : p.M - 1 - m0;
     aK[i] = c * 8;
     aOff[i] = (uint32_t(rr) * uint32_t(p.lda) + c * 8) * 2u;
-    aDst[i] = r * 128 + swzK(r, c) * 16;
+    if (i == 0)
+      aDst0 = r * 128 + swzK(r, c) * 16;
   }
 #pragma unroll
   for (int i = 0; i < B_PER_T; i++) {
@@ -709,17 +722,40 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(GemmParams p) {
       const int rr = n0 + r < p.N ? r : p.N - 1 - n0;
       bK[i] = c * 8;
       bOff[i] = (uint32_t(rr) * uint32_t(p.ldb) + c * 8) * 2u;
-      bDst[i] = r * 128 + swzK(r, c) * 16;
+      if (i == 0)
+        bDst0 = r * 128 + swzK(r, c) * 16;
     } else {
       const int cc = n0 + c * 8 < p.N ? c * 8 : p.N - 8 - n0;
       bK[i] = r;
       bOff[i] = (uint32_t(r) * uint32_t(p.ldb) + cc) * 2u;
-      bDst[i] = r * B_ROW_BYTES + swzN<BN>(r, c / 4) * 64 + (c % 4) * 16;
+      if (i == 0)
+        bDst0 = r * B_ROW_BYTES + swzN<BN>(r, c / 4) * 64 + (c % 4) * 16;
     }
   }
 
   half8 regA[DIST][A_PER_T], regB[DIST][B_PER_T];
+  // Slabs of this slice that lie inside [0, kEnd) entirely, and whether a
+  // partial one follows them (only the last slice of a ragged K has one).
+  const int nkFull = (kEnd - ktBegin * BK) / BK;
+  const bool hasTail = kEnd - ktBegin * BK > nkFull * BK;
+  const int ktLastFull = ktBegin + nkFull - 1;
+  // Full slab kt (requests past the last full slab fetch that one again).
   auto loadGlobal = [&](int kt, auto setC) {
+    constexpr int S = decltype(setC)::value;
+    const int k0 = (kt < ktLastFull ? kt : ktLastFull) * BK;
+    const uint32_t sA = uint32_t(k0) * 2u;
+    const uint32_t sB = B_NK ? sA : uint32_t(k0) * uint32_t(p.ldb) * 2u;
+#pragma unroll
+    for (int i = 0; i < A_PER_T; i++)
+      regA[S][i] = __builtin_bit_cast(
+          half8, __builtin_amdgcn_raw_buffer_load_b128(rsrcA, aOff[i], sA, 0));
+#pragma unroll
+    for (int i = 0; i < B_PER_T; i++)
+      regB[S][i] = __builtin_bit_cast(
+          half8, __builtin_amdgcn_raw_buffer_load_b128(rsrcB, bOff[i], sB, 0));
+  };
+  // Slab kt with a range test per vector (the partial slab).
+  auto loadGlobalChecked = [&](int kt, auto setC) {
     constexpr int S = decltype(setC)::value;
     const int k0 = kt * BK;
     const uint32_t sA = uint32_t(k0) * 2u;
@@ -741,10 +777,10 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(GemmParams p) {
     unsigned char *sB = sA + A_BYTES;
 #pragma unroll
     for (int i = 0; i < A_PER_T; i++)
-      *reinterpret_cast<half8 *>(sA + aDst[i]) = regA[S][i];
+      *reinterpret_cast<half8 *>(sA + aDst0 + i * DST_STEP) = regA[S][i];
 #pragma unroll
     for (int i = 0; i < B_PER_T; i++)
-      *reinterpret_cast<half8 *>(sB + bDst[i]) = regB[S][i];
+      *reinterpret_cast<half8 *>(sB + bDst0 + i * DST_STEP) = regB[S][i];
   };
 
   float16v acc[MI][NI];
@@ -834,8 +870,9 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(GemmParams p) {
   constexpr int NM = MI * NI;           // MFMAs per wavefront and k step
   constexpr int ST_STEPS = KSTEPS - 1;  // k steps that carry staging work
   half8 fa[2][MI], fb[2][NI];
-  const int nk = ktEnd - ktBegin;
-  // Moves vector v of register set S to LDS and refills it from slab kt.
+  const int nk = nkFull; // the pipelined loop walks the full slabs
+  // Moves vector v of register set S to LDS and refills it from full slab kt
+  // (already clamped to the last full slab by the caller).
   auto stageVec = [&](int stage, int kt, auto setC, auto vC) {
     constexpr int S = decltype(setC)::value;
     constexpr int V = decltype(vC)::value;
@@ -843,18 +880,17 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(GemmParams p) {
     unsigned char *sB = sA + A_BYTES;
     const int k0 = kt * BK;
     if constexpr (V < A_PER_T) {
-      *reinterpret_cast<half8 *>(sA + aDst[V]) = regA[S][V];
+      *reinterpret_cast<half8 *>(sA + aDst0 + V * DST_STEP) = regA[S][V];
       regA[S][V] = __builtin_bit_cast(
-          half8, __builtin_amdgcn_raw_buffer_load_b128(
-                     rsrcA, k0 + aK[V] < kEnd ? aOff[V] : kOob,
-                     uint32_t(k0) * 2u, 0));
+          half8, __builtin_amdgcn_raw_buffer_load_b128(rsrcA, aOff[V],
+                                                       uint32_t(k0) * 2u, 0));
     } else {
       constexpr int W = V - A_PER_T;
-      *reinterpret_cast<half8 *>(sB + bDst[W]) = regB[S][W];
+      *reinterpret_cast<half8 *>(sB + bDst0 + W * DST_STEP) = regB[S][W];
       regB[S][W] = __builtin_bit_cast(
           half8,
           __builtin_amdgcn_raw_buffer_load_b128(
-              rsrcB, k0 + bK[W] < kEnd ? bOff[W] : kOob,
+              rsrcB, bOff[W],
               B_NK ? uint32_t(k0) * 2u : uint32_t(k0) * uint32_t(p.ldb) * 2u,
               0));
     }
@@ -901,7 +937,8 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(GemmParams p) {
     constexpr bool kTail = decltype(tailC)::value;
     const int cur = i & 1;
     const bool more = !kTail || i + 1 < nk;
-    const int ktNext = ktBegin + i + 1 + DIST;
+    const int ktWant = ktBegin + i + 1 + DIST;
+    const int ktNext = ktWant < ktLastFull ? ktWant : ktLastFull;
     staticFor<KSTEPS>([&](auto kkC) {
       constexpr int kk = decltype(kkC)::value;
       constexpr int V0 = kk < ST_STEPS ? kk * NV / ST_STEPS : NV;
@@ -928,6 +965,22 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(GemmParams p) {
       }
     });
   };
+  if (hasTail) {
+    // The partial slab, unpipelined: it is one slab of a ragged problem.
+    using Set0 = std::integral_constant<int, 0>;
+    loadGlobalChecked(ktBegin + nkFull, Set0{});
+    storeLds(0, Set0{});
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < KSTEPS; kk++) {
+      loadFrags(0, kk, fa[0], fb[0]);
+#pragma unroll
+      for (int m = 0; m < NM; m++)
+        acc[m / NI][m % NI] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+            fb[0][m % NI], fa[0][m / NI], acc[m / NI][m % NI], 0, 0, 0);
+    }
+    __syncthreads(); // buffer 0 is rewritten by the first full slab
+  }
   if (nk > 0) {
     staticFor<DIST>(
         [&](auto d) { loadGlobal(ktBegin + decltype(d)::value, d); });
