@@ -65,6 +65,7 @@ typedef _Float16 half4 __attribute__((ext_vector_type(4)));
 typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 typedef float float16v __attribute__((ext_vector_type(16)));
 typedef float float4v __attribute__((ext_vector_type(4)));
+typedef float float2v __attribute__((ext_vector_type(2)));
 typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
 typedef short short4v __attribute__((ext_vector_type(4)));
 
@@ -85,7 +86,19 @@ struct GemmParams {
   float alpha, beta;
   int tilesM, tilesN;
   int kTilesPerSlice;
+  // layer-norm pair (kEpiRowStats / kEpiRowAffine kernels only)
+  float *rowStatPartials;
+  const _Float16 *rowScale;
+  const _Float16 *rowShift;
+  const float *colSum;
+  int colSumSlices;
 };
+
+// Epilogue codes beyond the three activations of the manifest kernels: linear
+// output plus row-statistic partial sums, and linear output of a per-row
+// affine transform of A folded into the accumulator.
+constexpr int kEpiRowStats = 3;
+constexpr int kEpiRowAffine = 4;
 
 // GELU(x) = 0.5 x (1 + erf(x / sqrt 2)) = max(x, 0) - 0.5 |x| erfc(|x| / sqrt 2)
 // (x >= 0: 1 + erf = 2 - erfc; x < 0: 1 + erf = erfc(|z|); no cancellation on
@@ -225,6 +238,22 @@ epilogueStoreLds(const GemmParams &p, float16v (&acc)[MI][NI], int m0, int n0,
   const int n = n0 + waveN * WTN + cc;
   // 16-byte accesses need rows of C and D that start 16-byte aligned
   const bool vec16 = p.ldd % 8 == 0 && (!useC || p.ldc % 8 == 0);
+  // Row-affine kernels: column sums of B for this lane's 8 columns (the same
+  // columns in every pass), summed over the slices they were computed in.
+  float cs[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  if constexpr (EPI == kEpiRowAffine) {
+    if (n < p.N)
+      for (int sl = 0; sl < p.colSumSlices; sl++) {
+        const float4v *src = reinterpret_cast<const float4v *>(
+            p.colSum + int64_t(sl) * p.N + n);
+        const float4v a = src[0], b = src[1];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          cs[e] += a[e];
+          cs[e + 4] += b[e];
+        }
+      }
+  }
   __syncthreads();
 #pragma unroll
   for (int i = 0; i < MI; i++) {
@@ -247,6 +276,7 @@ epilogueStoreLds(const GemmParams &p, float16v (&acc)[MI][NI], int m0, int n0,
       const float4v hi =
           *reinterpret_cast<const float4v *>(mine + r * ROW_B + cc * 4 + 16);
       const int m = m0 + waveM * WTM + i * 32 + r;
+      float rowSum = 0.f, rowSq = 0.f;
       if (m < p.M && n < p.N) {
         const _Float16 *cPtr = p.C + int64_t(m % p.cRowPeriod) * p.ldc + n;
         _Float16 *dPtr = p.D + int64_t(m) * p.ldd + n;
@@ -269,13 +299,31 @@ epilogueStoreLds(const GemmParams &p, float16v (&acc)[MI][NI], int m0, int n0,
               }
           }
         }
+        float rowScale = 1.f, rowShift = 0.f;
+        if constexpr (EPI == kEpiRowAffine) {
+          rowScale = float(p.rowScale[m]);
+          rowShift = float(p.rowShift[m]);
+        }
         half8 o;
 #pragma unroll
         for (int e = 0; e < 8; e++) {
-          float v = p.alpha * (e < 4 ? lo[e] : hi[e - 4]);
+          float a = e < 4 ? lo[e] : hi[e - 4];
+          if constexpr (EPI == kEpiRowAffine)
+            a = fmaf(rowScale, a, rowShift * cs[e]);
+          float v = p.alpha * a;
           if (useC)
             v += p.beta * c[e];
           o[e] = _Float16(activate<EPI>(v));
+        }
+        if constexpr (EPI == kEpiRowStats) {
+          // statistics of the values as stored
+#pragma unroll
+          for (int e = 0; e < 8; e++)
+            if (n + e < p.N) {
+              const float x = float(o[e]);
+              rowSum += x;
+              rowSq = fmaf(x, x, rowSq);
+            }
         }
         if (vec16) {
           *reinterpret_cast<half8 *>(dPtr) = o;
@@ -288,6 +336,23 @@ epilogueStoreLds(const GemmParams &p, float16v (&acc)[MI][NI], int m0, int n0,
               ov[1] = o[e + 1];
               *reinterpret_cast<half2v *>(dPtr + e) = ov;
             }
+        }
+      }
+      if constexpr (EPI == kEpiRowStats) {
+        // the LPR lanes of a row hold its WTN columns: one partial per row and
+        // wavefront column
+#pragma unroll
+        for (int off = LPR / 2; off > 0; off >>= 1) {
+          rowSum += __shfl_xor(rowSum, off, kWave);
+          rowSq += __shfl_xor(rowSq, off, kWave);
+        }
+        if (lane % LPR == 0 && m < p.M) {
+          const int piece = (n0 + waveN * WTN) / WTN;
+          float2v st;
+          st[0] = rowSum;
+          st[1] = rowSq;
+          *reinterpret_cast<float2v *>(p.rowStatPartials +
+                                       (int64_t(piece) * p.M + m) * 2) = st;
         }
       }
     }
@@ -1281,6 +1346,81 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmStagedKernel(GemmParams p) 
   epilogueStore<MI, NI, WTM, WTN, EPI, VEC>(p, acc, m0, n0, waveM, waveN, lane);
 }
 
+// ------------------------------------------------------- layer-norm pair --
+// Row-statistic partials [pieces][M] (sum, sum of squares) -> var / mean in the
+// form the pair exchanges (Layernorm.h:166-192 of the reference: the second
+// moment minus the squared mean, no shift).  Four lanes per row, 16 apart in
+// the wavefront so that 16 neighbouring lanes read 16 neighbouring rows; each
+// takes every fourth piece, four loads in flight.
+__global__ __launch_bounds__(256) void rowStatsFinalizeKernel(
+    const float *__restrict__ partials, int pieces, int M, int N, float eps,
+    _Float16 *__restrict__ var, _Float16 *__restrict__ mean) {
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int q = lane / 16;
+  const int m = (blockIdx.x * 4 + wave) * 16 + lane % 16;
+  const int mc = m < M ? m : M - 1;
+  float s = 0.f, sq = 0.f;
+  for (int pc = q; pc < pieces; pc += 16) {
+    float2v v[4];
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+      const int pu = pc + 4 * u;
+      v[u] = pu < pieces ? *reinterpret_cast<const float2v *>(
+                               partials + (int64_t(pu) * M + mc) * 2)
+                         : float2v{0.f, 0.f};
+    }
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+      s += v[u][0];
+      sq += v[u][1];
+    }
+  }
+  s += __shfl_xor(s, 16, kWave);
+  sq += __shfl_xor(sq, 16, kWave);
+  s += __shfl_xor(s, 32, kWave);
+  sq += __shfl_xor(sq, 32, kWave);
+  if (q == 0 && m < M) {
+    const float mu = s / float(N);
+    const float rstd = 1.0f / sqrtf(sq / float(N) - mu * mu + eps);
+    var[m] = _Float16(rstd);
+    mean[m] = _Float16(-mu * rstd);
+  }
+}
+
+// Partial column sums of row-major B [K, N]: workgroup (x, y) sums rows
+// [y * kPer, (y + 1) * kPer) of columns [32 x, 32 x + 32) into out[y][n].  A
+// thread reads 8 columns of every 64th row; the 64 row phases meet in LDS.
+__global__ __launch_bounds__(256) void colSumKernel(
+    const _Float16 *__restrict__ B, int64_t ldb, int K, int N, int kPer,
+    float *__restrict__ out) {
+  __shared__ float part[64][33];
+  const int tid = threadIdx.x;
+  const int cg = tid % 4, ph = tid / 4;
+  const int n = blockIdx.x * 32 + cg * 8;
+  const int kBegin = blockIdx.y * kPer;
+  const int kEnd = kBegin + kPer < K ? kBegin + kPer : K;
+  float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  if (n < N) {
+#pragma unroll 4
+    for (int k = kBegin + ph; k < kEnd; k += 64) {
+      const half8 v = *reinterpret_cast<const half8 *>(B + int64_t(k) * ldb + n);
+#pragma unroll
+      for (int e = 0; e < 8; e++)
+        acc[e] += float(v[e]);
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < 8; e++)
+    part[ph][cg * 8 + e] = acc[e];
+  __syncthreads();
+  if (tid < 32 && blockIdx.x * 32 + tid < N) {
+    float sum = 0.f;
+    for (int r = 0; r < 64; r++)
+      sum += part[r][tid];
+    out[int64_t(blockIdx.y) * N + blockIdx.x * 32 + tid] = sum;
+  }
+}
+
 // ------------------------------------------------------------ kernel table --
 struct LaunchPlan {
   GemmParams p;
@@ -1305,6 +1445,11 @@ Status planLaunch(const GemmProblem &pr, LaunchPlan *plan) {
   p.cRowPeriod = int(pr.cRowPeriod > 0 ? pr.cRowPeriod : 1);
   p.alpha = pr.alpha;
   p.beta = pr.beta;
+  p.rowStatPartials = pr.rowStatPartials;
+  p.rowScale = pr.rowScale;
+  p.rowShift = pr.rowShift;
+  p.colSum = pr.colSum;
+  p.colSumSlices = pr.colSumSlices;
   p.tilesM = int((pr.M + BM - 1) / BM);
   p.tilesN = int((pr.N + BN - 1) / BN);
   const int kTiles = int((pr.K + BK - 1) / BK);
@@ -1537,6 +1682,33 @@ const KernelEntry kKernels[] = {
 };
 constexpr int kNumKernels = sizeof(kKernels) / sizeof(kKernels[0]);
 
+// Tiles the layer-norm pair kernels exist in (square, `edge` on a side, a
+// wavefront covering `pieceWidth` columns); `likeKernel` picks the nearest.
+struct FusedTile {
+  int edge;
+  int pieceWidth;
+};
+FusedTile fusedTileFor(int likeKernel) {
+  const GemmKernelInfo &like = kKernels[likeKernel].info;
+  const int area = like.tileM * like.tileN;
+  if (area >= 256 * 256)
+    return {256, 64};
+  if (area >= 128 * 128)
+    return {128, 32};
+  return {64, 32};
+}
+template <int EPI>
+Status launchFusedTile(int likeKernel, const GemmProblem &p, hipStream_t s) {
+  switch (fusedTileFor(likeKernel).edge) {
+  case 256:
+    return launchPipe<256, 256, 2, 4, 1, EPI, false>(p, s);
+  case 128:
+    return launchPipe<128, 128, 2, 4, 2, EPI, false>(p, s);
+  default:
+    return launchPipe<64, 64, 2, 2, 2, EPI, false>(p, s);
+  }
+}
+
 inline bool aligned16(const void *p) {
   return (reinterpret_cast<uintptr_t>(p) & 15) == 0;
 }
@@ -1583,6 +1755,68 @@ Status launchGemm(int idx, const GemmProblem &p, hipStream_t s) {
   if (p.M == 0 || p.N == 0)
     return Status::kSuccess;
   return (p.bIsNK ? k.nt : k.nn)(p, s);
+}
+
+bool fusedGemmFits(const GemmProblem &p) {
+  return !p.bIsNK && p.M > 0 && p.N > 0 && p.K > 0 &&
+         p.M < (int64_t(1) << 31) && p.N < (int64_t(1) << 31) &&
+         p.K < (int64_t(1) << 31) && p.K % 8 == 0 && p.N % 8 == 0 &&
+         p.lda % 8 == 0 && p.ldb % 8 == 0 && p.ldd % 8 == 0 &&
+         aligned16(p.A) && aligned16(p.B) && aligned16(p.D) &&
+         (p.beta == 0.f || (p.C && p.ldc % 8 == 0 && aligned16(p.C)));
+}
+
+Status launchGemmRowStats(int likeKernel, const GemmProblem &p, _Float16 *var,
+                          _Float16 *mean, float eps, hipStream_t s) {
+  HOM_CHECK_RET(likeKernel >= 0 && likeKernel < kNumKernels && fusedGemmFits(p),
+                Status::kInvalidArgument,
+                "gemm + row statistics: problem does not fit the fused kernels");
+  // every tile writes all of its wavefront columns, also those past N
+  const FusedTile t = fusedTileFor(likeKernel);
+  const int pieces =
+      int((p.N + t.edge - 1) / t.edge) * (t.edge / t.pieceWidth);
+  float *partials = static_cast<float *>(
+      scratch(kTemp, size_t(pieces) * size_t(p.M) * 2 * sizeof(float), false));
+  if (!partials)
+    return Status::kInternal;
+  GemmProblem q = p;
+  q.splitK = 1;
+  q.rowStatPartials = partials;
+  Status st = launchFusedTile<kEpiRowStats>(likeKernel, q, s);
+  if (st != Status::kSuccess)
+    return st;
+  rowStatsFinalizeKernel<<<dim3((unsigned)((p.M + 63) / 64)), dim3(256), 0,
+                           s>>>(partials, pieces, int(p.M), int(p.N), eps, var,
+                                mean);
+  HOM_HIP_RET(hipGetLastError(), Status::kInternal);
+  return Status::kSuccess;
+}
+
+Status launchGemmRowAffine(int likeKernel, const GemmProblem &p,
+                           const _Float16 *var, const _Float16 *mean,
+                           hipStream_t s) {
+  HOM_CHECK_RET(likeKernel >= 0 && likeKernel < kNumKernels && fusedGemmFits(p),
+                Status::kInvalidArgument,
+                "layernorm + gemm: problem does not fit the fused kernels");
+  // 512 rows of B per column-sum workgroup, at most 16 slices
+  int slices = int((p.K + 511) / 512);
+  if (slices > 16)
+    slices = 16;
+  const int kPer = int((p.K + slices - 1) / slices);
+  float *colSum = static_cast<float *>(
+      scratch(kTemp, size_t(slices) * size_t(p.N) * sizeof(float), false));
+  if (!colSum)
+    return Status::kInternal;
+  colSumKernel<<<dim3((unsigned)((p.N + 31) / 32), (unsigned)slices), dim3(256),
+                 0, s>>>(p.B, p.ldb, int(p.K), int(p.N), kPer, colSum);
+  HOM_HIP_RET(hipGetLastError(), Status::kInternal);
+  GemmProblem q = p;
+  q.splitK = 1;
+  q.rowScale = var;
+  q.rowShift = mean;
+  q.colSum = colSum;
+  q.colSumSlices = slices;
+  return launchFusedTile<kEpiRowAffine>(likeKernel, q, s);
 }
 
 } // namespace hom

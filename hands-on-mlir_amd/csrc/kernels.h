@@ -76,6 +76,19 @@ struct GemmProblem {
   float alpha, beta;
   bool bIsNK;
   int splitK;
+  // Layer-norm pair, used by launchGemmRowStats / launchGemmRowAffine only
+  // (null otherwise).
+  // Out: (sum, sum of squares) of every stored row piece, one float2 per row
+  // and per wavefront column of the tile grid, [pieces][M].
+  float *rowStatPartials;
+  // In: D = alpha * (rowScale[m] * (A B)[m,n] + rowShift[m] * colSum[n]) +
+  // beta * C, i.e. the product of the row-normalised A with B without ever
+  // forming the normalised A.  colSum holds colSumSlices partial column sums
+  // of B, [slices][N].
+  const _Float16 *rowScale;
+  const _Float16 *rowShift;
+  const float *colSum;
+  int colSumSlices;
 };
 
 struct GemmKernelInfo {
@@ -96,5 +109,23 @@ int gemmKernelCount();
 const GemmKernelInfo &gemmKernelInfo(int idx);
 // Validates alignment/split-K against the kernel and launches it.
 Status launchGemm(int idx, const GemmProblem &p, hipStream_t s);
+
+// The layer-norm pair with the normalisation folded into the two GEMMs'
+// epilogues.  Both need the vector alignment class (K, N and the leading
+// dimensions multiples of 8, B row-major) -- fusedGemmFits() says whether a
+// problem qualifies -- and `likeKernel`, a manifest index whose tile size they
+// imitate.
+bool fusedGemmFits(const GemmProblem &p);
+// D = alpha A B + beta C, plus per-row statistics of the stored D:
+// var[m] = 1 / sqrt(E[d^2] - E[d]^2 + eps), mean[m] = -E[d] * var[m]
+// (the statistic is accumulated in the epilogue, a second small kernel turns
+// the per-tile partial sums into var / mean).
+Status launchGemmRowStats(int likeKernel, const GemmProblem &p, _Float16 *var,
+                          _Float16 *mean, float eps, hipStream_t s);
+// D = alpha (A * var[m] + mean[m]) B + beta C, computed as
+// alpha (var[m] (A B) + mean[m] colsum(B)) + beta C.
+Status launchGemmRowAffine(int likeKernel, const GemmProblem &p,
+                           const _Float16 *var, const _Float16 *mean,
+                           hipStream_t s);
 
 } // namespace hom

@@ -2,6 +2,7 @@
 symbol the header declares, and rejects bad arguments before touching the GPU."""
 import ctypes
 import importlib
+import json
 import os
 import re
 import subprocess
@@ -86,6 +87,35 @@ def test_select_returns_compatible_kernel(rt):
         elif N % 8:
             # even N: only the register-staged family reads rows that start at 4-byte boundaries
             assert align == 8 and "_64x2r" in name
+
+
+def test_selection_model_without_the_tuned_table():
+    """The timing model that answers for untuned shapes, asked about shapes the autotuner measured: it must land on
+    the tile class the measurements favour (its own process: the switch is read once)."""
+    code = r"""
+import ctypes, importlib, json, sys
+sys.path.insert(0, %r)
+rt = importlib.import_module("hands-on-mlir_amd.hom_runtime")
+lib = rt.load_runtime(); man = rt.manifest()
+idx, sk = ctypes.c_int64(), ctypes.c_int32()
+out = {}
+for shape in [(16384, 1024, 4096, 0), (16384, 4096, 1024, 1), (1024, 768, 768, 0), (1024, 2304, 768, 0),
+              (128, 1024, 4096, 0), (1024, 30522, 768, 0), (4096, 768, 3072, 0)]:
+    lib.homGemmSelect(*shape, ctypes.byref(idx), ctypes.byref(sk))
+    out["x".join(map(str, shape))] = [man[idx.value][1], sk.value]
+print(json.dumps(out))
+""" % ROOT
+    env = dict(os.environ, HOM_GEMM_IGNORE_TUNED_TABLE="1")
+    res = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=120)
+    assert res.returncode == 0, res.stderr
+    picks = json.loads(res.stdout.strip().splitlines()[-1])
+    assert "_256x256_64x2r1_w2x4_" in picks["16384x1024x4096x0"][0]
+    assert "_256x256_64x2r1_w2x4_" in picks["16384x4096x1024x1"][0] and picks["16384x4096x1024x1"][0].endswith("_gelu")
+    assert "_64x64_64x2r2_" in picks["1024x768x768x0"][0] and picks["1024x768x768x0"][1] == 1
+    assert "_128x128_64x2r2_w2x4_" in picks["1024x2304x768x0"][0]
+    assert "_128x128_64x2r2_w2x4_" in picks["4096x768x3072x0"][0]
+    assert "_64x64_" in picks["128x1024x4096x0"][0] and picks["128x1024x4096x0"][1] > 1    # skinny: split-K
+    assert "_64x2r" in picks["1024x30522x768x0"][0] and picks["1024x30522x768x0"][1] == 1  # even N: pipe family
 
 
 # ---- argument checking: runs without a GPU because every check precedes the

@@ -349,6 +349,48 @@ def test_ln_gemm_pair(gpu, rt, oracle, literals):
     assert_close(host(out)[0], ln @ c[0].astype(np.float64), rtol=1e-2, atol=2e-2)
 
 
+@pytest.mark.parametrize("Mp,N1,K1,N2,beta", [
+    (1024, 768, 768, 768, 0.0),      # 64x64 tiles for both halves
+    (1024, 768, 768, 2304, 1.0),     # second half on 128x128 tiles, residual source
+    (4096, 1024, 256, 2304, 0.0),    # second half on 256x256 tiles
+    (1000, 776, 264, 520, 1.0),      # ragged rows and columns (still multiples of 8)
+    (100, 250, 72, 30, 0.0),         # N not a multiple of 8: the unfused kernels
+])
+def test_ln_gemm_pair_shapes(gpu, rt, oracle, Mp, N1, K1, N2, beta):
+    """GEMM + row statistics, then GEMM of the row-normalised result, at sizes that reach every fused tile
+    (LayernormGemmRunner.h:17-361).  The second product is checked against the affine row transform applied in
+    fp64 with the var/mean values the first call stored."""
+    M = rt.MemRef.from_tensor
+    g = np.random.default_rng(Mp + N1 + N2)
+    a = g.standard_normal((1, Mp, K1)).astype(np.float16)
+    b = (g.standard_normal((1, K1, N1)) * 0.05).astype(np.float16)
+    c = (g.standard_normal((1, N1, N2)) * 0.05).astype(np.float16)
+    # rows with a mean well away from zero make the colsum term matter
+    src = (g.standard_normal((1, Mp, N1)) + 1.5).astype(np.float16)
+    eps = 1e-5
+    ta, tb, tc = dev(a), dev(b), dev(c)
+    d1 = dev(src) if beta else torch.zeros((1, Mp, N1), dtype=torch.float16, device="cuda")
+    var = torch.zeros((1, Mp, 1), dtype=torch.float16, device="cuda")
+    mean = torch.zeros((1, Mp, 1), dtype=torch.float16, device="cuda")
+    gpu.cutlassGemmWithVarMeanF16(*M(ta).args(), *M(tb).args(), *M(d1).args(), *M(d1).args(),
+                                  *M(var).args(), *M(mean).args(), 1.0, beta, 0, eps)
+    want_d1 = oracle.gemm(a[0], b[0], src[0] if beta else None, beta=beta)
+    got_d1 = host(d1)[0]
+    assert_close(got_d1, want_d1, **GEMM_TOL, what="first product")
+    v, m = oracle.row_stats(got_d1.astype(np.float32), eps)
+    assert_close(host(var).ravel(), v, rtol=2e-3, atol=1e-3, what="var")
+    assert_close(host(mean).ravel(), m, rtol=2e-3, atol=2e-3, what="mean")
+
+    res = (g.standard_normal((1, Mp, N2))).astype(np.float16)
+    out = dev(res) if beta else torch.zeros((1, Mp, N2), dtype=torch.float16, device="cuda")
+    gpu.cutlassLayernormGemmF16(*M(d1).args(), *M(tc).args(), *M(out).args(), *M(out).args(),
+                                *M(var).args(), *M(mean).args(), 1.0, beta, 0)
+    ln = got_d1.astype(np.float64) * host(var).reshape(Mp, 1).astype(np.float64) \
+        + host(mean).reshape(Mp, 1).astype(np.float64)
+    want = ln @ c[0].astype(np.float64) + (beta * res[0].astype(np.float64) if beta else 0.0)
+    assert_close(host(out)[0], want, **GEMM_TOL, what="second product")
+
+
 # --------------------------------------------------------------- attention --
 def run_attention(gpu, rt, qkv, lens, heads, scale):
     M = rt.MemRef.from_tensor
