@@ -50,6 +50,21 @@ __device__ __forceinline__ int swzV(int k, int group) {
   return group ^ ((k >> 1) & 1);
 }
 
+// Combine a value with the one in lane ^ 32.  v_permlane32_swap exchanges the
+// upper half of its first operand with the lower half of its second; given
+// the same value twice it returns (lower-half values, upper-half values) in
+// every lane pair -- one VALU instruction where a shuffle is an LDS round trip.
+__device__ __forceinline__ float pairMax(float v) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v),
+                                                  __float_as_uint(v), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float pairSum(float v) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v),
+                                                  __float_as_uint(v), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
 template <int NW>
 __global__ __launch_bounds__(NW *kWave) void bertAttentionKernel(
     const _Float16 *__restrict__ qkv, const int32_t *__restrict__ cu,
@@ -227,7 +242,7 @@ __global__ __launch_bounds__(NW *kWave) void bertAttentionKernel(
 #pragma unroll
         for (int e = 0; e < 16; e++)
           blockMax = fmaxf(blockMax, accS[sb][e]);
-      blockMax = fmaxf(blockMax, __shfl_xor(blockMax, 32, kWave));
+      blockMax = pairMax(blockMax);
       const float newMax = fmaxf(rowMax, blockMax);
       // Every block that is visited has at least one valid key, so newMax is
       // finite and the differences below are never inf - inf.
@@ -243,7 +258,7 @@ __global__ __launch_bounds__(NW *kWave) void bertAttentionKernel(
           accS[sb][e] = pv;
           blockSum += pv;
         }
-      blockSum += __shfl_xor(blockSum, 32, kWave);
+      blockSum = pairSum(blockSum);
       rowSum = rowSum * corr + blockSum;
       rowMax = newMax;
 #pragma unroll

@@ -136,6 +136,25 @@ template <int EPI> __device__ __forceinline__ float activate(float v) {
   return v;
 }
 
+// Sum over groups of N consecutive lanes (N = 4, 8 or 16, groups aligned to
+// N) with data-parallel-primitive adds: quad permutes exchange lanes ^1 and ^2,
+// the half-row and row mirrors pair each lane with one of the other quad /
+// the other half of its 16-lane row.  No LDS round trips, unlike shuffles.
+template <int CTRL> __device__ __forceinline__ float addDpp(float v) {
+  return v + __int_as_float(__builtin_amdgcn_update_dpp(
+                 0, __float_as_int(v), CTRL, 0xf, 0xf, false));
+}
+template <int N> __device__ __forceinline__ float sumAcrossLanes(float v) {
+  static_assert(N == 4 || N == 8 || N == 16, "group size");
+  v = addDpp<0xB1>(v); // quad_perm [1,0,3,2]
+  v = addDpp<0x4E>(v); // quad_perm [2,3,0,1]
+  if (N >= 8)
+    v = addDpp<0x141>(v); // row_half_mirror
+  if (N >= 16)
+    v = addDpp<0x140>(v); // row_mirror
+  return v;
+}
+
 // XCD-contiguous tile id for this workgroup.
 __device__ __forceinline__ int tileForBlock(int nTiles, int pid) {
   const int q = nTiles / kNumXcd, r = nTiles % kNumXcd;
@@ -341,11 +360,8 @@ epilogueStoreLds(const GemmParams &p, float16v (&acc)[MI][NI], int m0, int n0,
       if constexpr (EPI == kEpiRowStats) {
         // the LPR lanes of a row hold its WTN columns: one partial per row and
         // wavefront column
-#pragma unroll
-        for (int off = LPR / 2; off > 0; off >>= 1) {
-          rowSum += __shfl_xor(rowSum, off, kWave);
-          rowSq += __shfl_xor(rowSq, off, kWave);
-        }
+        rowSum = sumAcrossLanes<LPR>(rowSum);
+        rowSq = sumAcrossLanes<LPR>(rowSq);
         if (lane % LPR == 0 && m < p.M) {
           const int piece = (n0 + waveN * WTN) / WTN;
           float2v st;
@@ -1798,8 +1814,9 @@ Status launchGemmRowAffine(int likeKernel, const GemmProblem &p,
   HOM_CHECK_RET(likeKernel >= 0 && likeKernel < kNumKernels && fusedGemmFits(p),
                 Status::kInvalidArgument,
                 "layernorm + gemm: problem does not fit the fused kernels");
-  // 512 rows of B per column-sum workgroup, at most 16 slices
-  int slices = int((p.K + 511) / 512);
+  // 128 rows of B per column-sum workgroup (two 16-byte loads per lane), at
+  // most 16 slices
+  int slices = int((p.K + 127) / 128);
   if (slices > 16)
     slices = 16;
   const int kPer = int((p.K + slices - 1) / slices);

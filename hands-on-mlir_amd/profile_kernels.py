@@ -6,6 +6,9 @@ what:  gemm1      FFN1 GEMM + bias + tanh-GELU, M=1024 K=768 N=3072 (tuned kerne
        gemm5      BERT-large FFN2 GEMM, M=16384 K=4096 N=1024
        layernorm  in-place layer norm, 16384 x 1024
        attention  packed-QKV attention, b8 s128 h12
+       lnpair     the layer-norm pair at BERT-large size: GEMM + row statistics
+                  16384x1024x1024, then the GEMM of the normalised rows
+                  16384x4096x1024, next to the two plain GEMMs
        copy       plain device copy of 256 MiB (counter calibration: reads and
                   writes exactly 268435456 bytes each)
 Each call goes through the C-ABI via the C++ driver's timing helpers.
@@ -38,6 +41,26 @@ def main():
     elif what == "attention":
         lens = (ctypes.c_int32 * 8)(83, 128, 57, 101, 32, 120, 64, 99)
         print(f"attention b8 s128 h12: {drv.homTimeAttention(8, 128, 12, lens, iters, 3) * 1e3:.2f} us")
+    elif what == "lnpair":
+        import torch
+        M = rt.MemRef.from_tensor
+        g = torch.Generator(device="cuda").manual_seed(0)
+        rnd = lambda *shape, scale=1.0: (torch.randn(shape, device="cuda", generator=g) * scale).half()
+        x, w1, w2 = rnd(1, 16384, 1024), rnd(1, 1024, 1024, scale=0.03), rnd(1, 1024, 4096, scale=0.03)
+        d1 = torch.zeros((1, 16384, 1024), dtype=torch.float16, device="cuda")
+        d2 = torch.zeros((1, 16384, 4096), dtype=torch.float16, device="cuda")
+        var = torch.zeros((1, 16384, 1), dtype=torch.float16, device="cuda")
+        mean = torch.zeros_like(var)
+        mx, mw1, mw2, md1, md2, mv, mm = (M(t) for t in (x, w1, w2, d1, d2, var, mean))
+        for _ in range(iters):
+            lib.cutlassGemmF16(*mx.args(), False, *mw1.args(), False, *md1.args(), *md1.args(), 0, 1.0, 0.0, 0, 1)
+            lib.cutlassGemmF16(*md1.args(), False, *mw2.args(), False, *md2.args(), *md2.args(), 0, 1.0, 0.0, 0, 1)
+            lib.cutlassGemmWithVarMeanF16(*mx.args(), *mw1.args(), *md1.args(), *md1.args(), *mv.args(), *mm.args(),
+                                          1.0, 0.0, 0, 1e-5)
+            lib.cutlassLayernormGemmF16(*md1.args(), *mw2.args(), *md2.args(), *md2.args(), *mv.args(), *mm.args(),
+                                        1.0, 0.0, 0)
+        torch.cuda.synchronize()
+        print("ln pair 16384x1024x1024 -> 16384x4096x1024 x", iters)
     elif what == "copy":
         import torch
         src = torch.ones(128 * 1024 * 1024, dtype=torch.float16, device="cuda")

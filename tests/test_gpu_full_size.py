@@ -1,0 +1,167 @@
+"""The BERT-large kernel shapes (M = 32 x 512 = 16384 rows) through the C-ABI.
+
+The oracle is too slow for whole tensors of this size, so each operator is checked
+(a) against the oracle on a sample of rows / (batch, head) pairs, which touches
+every tile column and a spread of tile rows, and (b) through properties that hold
+for the whole tensor whatever its size: column-sum checksums for GEMM, constant-V
+and key-permutation invariance for attention, idempotence and unit statistics for
+layer norm, commutativity for add.  Tolerances are the ones of test_gpu_parity.
+"""
+import importlib
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+GEMM_TOL = dict(rtol=1e-3, atol=1e-2)
+LN_TOL = dict(rtol=2e-3, atol=1e-3)
+ROWS = 32 * 512
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def host(t):
+    torch.cuda.synchronize()
+    return t.cpu().numpy()
+
+
+def assert_close(got, want, rtol, atol, what=""):
+    got = np.asarray(got, np.float64)
+    want = np.asarray(want, np.float64)
+    err = np.abs(got - want)
+    bad = err > atol + rtol * np.abs(want)
+    assert not bad.any(), (f"{what}: {bad.sum()} of {bad.size} outside rtol={rtol} atol={atol}; "
+                           f"max abs err {err.max():.3e} at {np.unravel_index(err.argmax(), err.shape)}")
+
+
+def sample_rows(g, rows, count=48):
+    """First and last rows, rows either side of 256-row tile edges, and random ones."""
+    fixed = [0, 1, 255, 256, 257, rows // 2 - 1, rows // 2, rows - 257, rows - 256, rows - 1]
+    return np.unique(np.concatenate([fixed, g.integers(0, rows, size=count - len(fixed))]))
+
+
+@pytest.mark.parametrize("N,K,act,beta", [
+    (4096, 1024, 1, 0.0),   # FFN1 + GELU-erf
+    (1024, 4096, 0, 1.0),   # FFN2 + residual, in place
+    (3072, 1024, 0, 0.0),   # QKV projection
+])
+def test_gemm_bert_large_shapes(gpu, rt, oracle, N, K, act, beta):
+    M = rt.MemRef.from_tensor
+    g = np.random.default_rng(N + K)
+    a = g.standard_normal((32, 512, K), dtype=np.float32).astype(np.float16)
+    b = (g.standard_normal((1, K, N), dtype=np.float32) * 0.03).astype(np.float16)
+    res = g.standard_normal((32, 512, N), dtype=np.float32).astype(np.float16)
+    ta, tb = dev(a), dev(b)
+    td = dev(res) if beta else torch.zeros((32, 512, N), dtype=torch.float16, device="cuda")
+    gpu.cutlassGemmF16(*M(ta).args(), False, *M(tb).args(), False, *M(td).args(), *M(td).args(),
+                       act, 1.0, beta, 0, 1)
+    got = host(td).reshape(ROWS, N)
+    rows = sample_rows(g, ROWS)
+    want = oracle.gemm(a.reshape(ROWS, K)[rows], b[0], res.reshape(ROWS, N)[rows] if beta else None,
+                       beta=beta, act="gelu_erf" if act else "linear")
+    assert_close(got[rows], want, **GEMM_TOL, what=f"sampled rows of 16384x{N}x{K}")
+    if not act:
+        # checksum over every row: sum_j D[i, j] = A[i, :] . rowsum(B) (+ sum_j C[i, j]); the
+        # stored values carry one fp16 rounding each (relative 2^-11, independent)
+        a64 = a.reshape(ROWS, K).astype(np.float64)
+        check = a64 @ b[0].astype(np.float64).sum(axis=1)
+        if beta:
+            check += res.reshape(ROWS, N).astype(np.float64).sum(axis=1)
+        got64 = got.astype(np.float64)
+        noise = 2.0 ** -11 * np.sqrt((got64 ** 2).sum(axis=1))
+        assert (np.abs(got64.sum(axis=1) - check) <= 6 * noise + 1e-3).all(), "row checksum"
+    assert np.isfinite(got.astype(np.float32)).all()
+
+
+def run_attention(gpu, rt, qkv, lens, heads, scale):
+    M = rt.MemRef.from_tensor
+    bs, seq, w = qkv.shape
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    tq, tc = dev(qkv), dev(cu)
+    out = torch.full((bs, seq, w // 3), 7.0, dtype=torch.float16, device="cuda")
+    gpu.nvteBertAttentionF16(*M(tq).args(), *M(tc).args(), *M(out).args(), scale, heads)
+    return host(out), cu
+
+
+def test_attention_bert_large_shape(gpu, rt, oracle):
+    bs, seq, heads = 32, 512, 16
+    g = np.random.default_rng(7)
+    qkv = g.standard_normal((bs, seq, 3 * heads * 64), dtype=np.float32).astype(np.float16)
+    lens = g.integers(1, seq + 1, size=bs).astype(np.int32)
+    lens[:4] = [512, 1, 511, 65]
+    got, cu = run_attention(gpu, rt, qkv, lens, heads, 0.125)
+    # oracle on a sample of sequences (all heads of each)
+    for b in (0, 1, 2, 3, 17, 31):
+        one_cu = np.array([0, lens[b]], np.int32)
+        want = oracle.attention(qkv[b:b + 1], one_cu, heads, 0.125)
+        assert_close(got[b:b + 1], want, **GEMM_TOL, what=f"attention sequence {b} (len {lens[b]})")
+    for b, n in enumerate(lens):
+        assert not got[b, n:].any(), "padded query rows must be zeros"
+
+    # rows of P sum to 1: a V that is constant over the keys comes out unchanged
+    v5 = qkv.reshape(bs, seq, 3, heads, 64).copy()
+    const = g.standard_normal((bs, 1, heads, 64), dtype=np.float32).astype(np.float16)
+    v5[:, :, 2] = const
+    out_c, _ = run_attention(gpu, rt, v5.reshape(bs, seq, -1), lens, heads, 0.125)
+    out_c = out_c.reshape(bs, seq, heads, 64)
+    for b, n in enumerate(lens):
+        assert_close(out_c[b, :n], np.broadcast_to(const[b], (n, heads, 64)), rtol=2e-3, atol=2e-3,
+                     what=f"constant V, sequence {b}")
+
+    # permuting the valid keys (K and V rows together) changes nothing but the summation order
+    perm5 = qkv.reshape(bs, seq, 3, heads, 64).copy()
+    for b, n in enumerate(lens):
+        p = g.permutation(n)
+        perm5[b, :n, 1:] = perm5[b, p, 1:]
+    out_p, _ = run_attention(gpu, rt, perm5.reshape(bs, seq, -1), lens, heads, 0.125)
+    assert_close(out_p, got, rtol=2e-3, atol=4e-3, what="key permutation")
+
+
+def test_layernorm_bert_large_shape(gpu, rt, oracle):
+    g = np.random.default_rng(11)
+    x = (g.standard_normal((32, 512, 1024), dtype=np.float32) * 1.7 + 0.4).astype(np.float16)
+    t = dev(x)
+    gpu.nvteLayernormF16(*rt.MemRef.from_tensor(t).args(), 1e-12)
+    once = host(t).reshape(ROWS, 1024)
+    rows = sample_rows(g, ROWS)
+    assert_close(once[rows], oracle.layernorm_f16(x.reshape(ROWS, 1024)[rows], 1e-12), **LN_TOL)
+    o64 = once.astype(np.float64)
+    assert np.abs(o64.mean(axis=1)).max() <= 2e-3
+    assert np.abs(o64.var(axis=1) - 1.0).max() <= 5e-3
+    gpu.nvteLayernormF16(*rt.MemRef.from_tensor(t).args(), 1e-12)   # idempotent up to rounding
+    assert_close(host(t).reshape(ROWS, 1024), once, **LN_TOL, what="layer norm twice")
+
+
+def test_elementwise_gather_cu_seqlens_bert_large_shapes(gpu, rt, oracle):
+    M = rt.MemRef.from_tensor
+    g = np.random.default_rng(13)
+    a = g.standard_normal((32, 512, 1024), dtype=np.float32).astype(np.float16)
+    b = g.standard_normal((32, 512, 1024), dtype=np.float32).astype(np.float16)
+    ta, tb = dev(a), dev(b)
+    ab, ba = torch.empty_like(ta), torch.empty_like(ta)
+    gpu.thrustElementwiseAddF16(*M(ta).args(), *M(tb).args(), *M(ab).args())
+    gpu.thrustElementwiseAddF16(*M(tb).args(), *M(ta).args(), *M(ba).args())
+    assert torch.equal(ab, ba)
+    rows = sample_rows(g, ROWS)
+    want = oracle.elementwise("add", a.reshape(ROWS, 1024)[rows], b.reshape(ROWS, 1024)[rows])
+    assert np.array_equal(host(ab).reshape(ROWS, 1024)[rows], want.astype(np.float16))
+
+    vocab = 30522
+    table = g.standard_normal((1, vocab, 1024), dtype=np.float32).astype(np.float16)
+    ids = g.integers(0, vocab, size=(32, 512)).astype(np.int64)
+    ids[0, :3] = [0, vocab - 1, 0]
+    tt, ti = dev(table), dev(ids)
+    out = torch.empty((32, 512, 1024), dtype=torch.float16, device="cuda")
+    gpu.thrustGatherF16(*M(ti).args(), *M(tt).args(), *M(out).args())
+    assert np.array_equal(host(out), table[0][ids])
+
+    lens = g.integers(0, 513, size=32)
+    mask = (np.arange(512)[None, :] < lens[:, None]).astype(np.int64)
+    tm = dev(mask)
+    cu = torch.empty(33, dtype=torch.int32, device="cuda")
+    gpu.thrustCuSeqLenI64(*M(tm).args(), *M(cu).args())
+    assert np.array_equal(host(cu), np.concatenate([[0], np.cumsum(lens)]).astype(np.int32))
