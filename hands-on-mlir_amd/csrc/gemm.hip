@@ -1429,9 +1429,21 @@ __global__ __launch_bounds__(256) void colSumKernel(
   for (int e = 0; e < 8; e++)
     part[ph][cg * 8 + e] = acc[e];
   __syncthreads();
+  // 64 phases -> 8 -> 1, every thread busy in the first step
+  {
+    const int c = tid % 32, grp = tid / 32;
+    float sum = 0.f;
+#pragma unroll
+    for (int r = 0; r < 8; r++)
+      sum += part[grp * 8 + r][c];
+    __syncthreads();
+    part[grp][c] = sum;
+  }
+  __syncthreads();
   if (tid < 32 && blockIdx.x * 32 + tid < N) {
     float sum = 0.f;
-    for (int r = 0; r < 64; r++)
+#pragma unroll
+    for (int r = 0; r < 8; r++)
       sum += part[r][tid];
     out[int64_t(blockIdx.y) * N + blockIdx.x * 32 + tid] = sum;
   }
