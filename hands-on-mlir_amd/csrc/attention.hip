@@ -66,7 +66,8 @@ __device__ __forceinline__ float pairSum(float v) {
 }
 
 template <int NW>
-__global__ __launch_bounds__(NW *kWave) void bertAttentionKernel(
+__global__ __launch_bounds__(NW *kWave)
+__attribute__((amdgpu_waves_per_eu(2, 3))) void bertAttentionKernel(
     const _Float16 *__restrict__ qkv, const int32_t *__restrict__ cu,
     _Float16 *__restrict__ out, int seq, int heads, float scale) {
   constexpr int kThreads = NW * kWave;
@@ -149,7 +150,8 @@ __global__ __launch_bounds__(NW *kWave) void bertAttentionKernel(
 #pragma unroll
     for (int e = 0; e < 16; e++)
       accO[d][e] = 0.f;
-  float rowMax = -INFINITY, rowSum = 0.f; // rowMax in raw (unscaled) score units
+  // rowMax: reference of the exponent, in raw (unscaled) score units
+  float rowMax = -INFINITY, rowSum = 0.f;
   const float scaleLog2e = scale * 1.44269504088896340736f;
 
   // Per-lane constants of the fragment addresses.
@@ -205,6 +207,16 @@ __global__ __launch_bounds__(NW *kWave) void bertAttentionKernel(
 
     for (int blk = 0; blk < live; blk += 64) {
       // ---- S^T = K Q^T for two 32-key sub-blocks ----
+      // All eight K fragments are requested before the first MFMA: read one
+      // at a time, each MFMA would wait out a full LDS round trip.
+      half8 fk[2][kHeadDim / 16];
+#pragma unroll
+      for (int sb = 0; sb < 2; sb++)
+#pragma unroll
+        for (int kk = 0; kk < kHeadDim / 16; kk++)
+          fk[sb][kk] = *reinterpret_cast<const half8 *>(
+              sK + (blk + sb * 32 + l32) * 128 + ((kk * 2 + hb) ^ swzLane) * 16);
+      __builtin_amdgcn_sched_barrier(0);
       float16v accS[2];
 #pragma unroll
       for (int sb = 0; sb < 2; sb++) {
@@ -212,12 +224,9 @@ __global__ __launch_bounds__(NW *kWave) void bertAttentionKernel(
         for (int e = 0; e < 16; e++)
           accS[sb][e] = 0.f;
 #pragma unroll
-        for (int kk = 0; kk < kHeadDim / 16; kk++) {
-          const half8 fk = *reinterpret_cast<const half8 *>(
-              sK + (blk + sb * 32 + l32) * 128 + ((kk * 2 + hb) ^ swzLane) * 16);
-          accS[sb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fk, fq[kk], accS[sb],
-                                                            0, 0, 0);
-        }
+        for (int kk = 0; kk < kHeadDim / 16; kk++)
+          accS[sb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fk[sb][kk], fq[kk],
+                                                            accS[sb], 0, 0, 0);
       }
       // accS[sb][e] is the raw score (before scaling) of query l32 against key
       //   key0 + blk + sb*32 + 8*(e/4) + 4*hb + e%4.
@@ -243,11 +252,28 @@ __global__ __launch_bounds__(NW *kWave) void bertAttentionKernel(
         for (int e = 0; e < 16; e++)
           blockMax = fmaxf(blockMax, accS[sb][e]);
       blockMax = pairMax(blockMax);
-      const float newMax = fmaxf(rowMax, blockMax);
-      // Every block that is visited has at least one valid key, so newMax is
-      // finite and the differences below are never inf - inf.
-      const float corr = __builtin_amdgcn_exp2f((rowMax - newMax) * scaleLog2e);
-      const float negMax = -newMax * scaleLog2e;
+      // The exponent's reference rowMax only has to keep p within range, it
+      // need not be the true maximum: it moves (and O and the running sum are
+      // rescaled, 96 vector instructions on the accumulators) only when some
+      // row of the wavefront has grown past it by more than kSlack in the
+      // exponent, i.e. p would exceed 2^kSlack.  The final O / rowSum cancels
+      // whatever reference was used.  With real score distributions that
+      // happens in the first block or two of a row and rarely afterwards.
+      // Every block that is visited has at least one valid key, so blockMax
+      // is finite and the differences below are never inf - inf.
+      constexpr float kSlack = 8.0f;
+      if (__any((blockMax - rowMax) * scaleLog2e > kSlack)) {
+        const float newMax = fmaxf(rowMax, blockMax);
+        const float corr = __builtin_amdgcn_exp2f((rowMax - newMax) * scaleLog2e);
+        rowSum *= corr;
+        rowMax = newMax;
+#pragma unroll
+        for (int d = 0; d < 2; d++)
+#pragma unroll
+          for (int e = 0; e < 16; e++)
+            accO[d][e] *= corr;
+      }
+      const float negMax = -rowMax * scaleLog2e;
       float blockSum = 0.f;
 #pragma unroll
       for (int sb = 0; sb < 2; sb++)
@@ -259,13 +285,7 @@ __global__ __launch_bounds__(NW *kWave) void bertAttentionKernel(
           blockSum += pv;
         }
       blockSum = pairSum(blockSum);
-      rowSum = rowSum * corr + blockSum;
-      rowMax = newMax;
-#pragma unroll
-      for (int d = 0; d < 2; d++)
-#pragma unroll
-        for (int e = 0; e < 16; e++)
-          accO[d][e] *= corr;
+      rowSum += blockSum;
 
       // ---- O^T += V^T P^T ----
 #pragma unroll
