@@ -160,6 +160,22 @@ __attribute__((amdgpu_waves_per_eu(2, 3))) void bertAttentionKernel(
   const int trCol = ((lane % 32) / 16) * 16 + (lane % 4) * 4;
   const int vSwz = (trRow >> 1) & 1;           // key bases are multiples of 4
 
+  // Staging without prefetch: thread t copies 16-byte vector t % 8 of rows
+  // t / 8 + i * kThreads / 8.  Both swizzles depend on row bits that the
+  // per-vector row step (a multiple of 16) leaves alone, so the LDS
+  // destinations are one base plus immediates.
+  const uint32_t rowBytes = uint32_t(tokStride) * 2u;
+  const uint32_t stageOff = uint32_t(tid / 8) * rowBytes + uint32_t(tid % 8) * 16u;
+  const int stageK = (tid / 8) * 128 + swzK(tid / 8, tid % 8) * 16;
+  const int stageV =
+      (tid / 8) * 128 + swzV(tid / 8, (tid % 8) / 4) * 64 + ((tid % 8) % 4) * 16;
+  const auto rsrcK = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<_Float16 *>(kBase), 0, int32_t(uint32_t(len) * rowBytes),
+      0x00020000);
+  const auto rsrcV = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<_Float16 *>(vBase), 0, int32_t(uint32_t(len) * rowBytes),
+      0x00020000);
+
   const int numChunks = (len + kChunk - 1) / kChunk; // uniform over the workgroup
   for (int ch = 0; ch < numChunks; ch++) {
     const int key0 = ch * kChunk;
@@ -187,18 +203,23 @@ __attribute__((amdgpu_waves_per_eu(2, 3))) void bertAttentionKernel(
         }
       }
     } else {
-      for (int v = tid; v < live * 8; v += kThreads) {
-        const int r = v / 8, c = v % 8;
-        half8 kv, vv;
+      // Whole chunk, no range tests: the descriptors end at row `len`, so rows
+      // past the sequence read as zero without touching memory.  All loads go
+      // out before the first LDS store; addresses are one add per vector.
+      half8 kv[VPT], vv[VPT];
+      const uint32_t chunkOff = stageOff + uint32_t(key0) * rowBytes;
 #pragma unroll
-        for (int e = 0; e < 8; e++)
-          kv[e] = vv[e] = _Float16(0);
-        if (key0 + r < len) {
-          kv = *reinterpret_cast<const half8 *>(kBase + int64_t(key0 + r) * tokStride + c * 8);
-          vv = *reinterpret_cast<const half8 *>(vBase + int64_t(key0 + r) * tokStride + c * 8);
-        }
-        *reinterpret_cast<half8 *>(sK + r * 128 + swzK(r, c) * 16) = kv;
-        *reinterpret_cast<half8 *>(sV + r * 128 + swzV(r, c / 4) * 64 + (c % 4) * 16) = vv;
+      for (int i = 0; i < VPT; i++) {
+        const uint32_t off = chunkOff + uint32_t(i * (kThreads / 8)) * rowBytes;
+        kv[i] = __builtin_bit_cast(
+            half8, __builtin_amdgcn_raw_buffer_load_b128(rsrcK, off, 0, 0));
+        vv[i] = __builtin_bit_cast(
+            half8, __builtin_amdgcn_raw_buffer_load_b128(rsrcV, off, 0, 0));
+      }
+#pragma unroll
+      for (int i = 0; i < VPT; i++) {
+        *reinterpret_cast<half8 *>(sK + stageK + i * (kThreads / 8) * 128) = kv[i];
+        *reinterpret_cast<half8 *>(sV + stageV + i * (kThreads / 8) * 128) = vv[i];
       }
     }
     if (kPrefetch && ch + 1 < numChunks)
@@ -359,6 +380,10 @@ Status launchBertAttentionF16(const _Float16 *qkv, const int32_t *cuSeqlens,
                 "attention: scale must be positive (got %g)", double(scale));
   HOM_CHECK_RET(bs < 65536 && heads < 65536 && seq < (int64_t(1) << 24),
                 Status::kInvalidArgument, "attention: shape out of range");
+  // K/V staging addresses a batch entry with 32-bit byte offsets
+  HOM_CHECK_RET(seq * 3 * heads * kHeadDim * 2 < (int64_t(1) << 31),
+                Status::kInvalidArgument,
+                "attention: one batch entry of QKV must be smaller than 2 GiB");
   HOM_CHECK_RET((reinterpret_cast<uintptr_t>(qkv) & 15) == 0 &&
                     (reinterpret_cast<uintptr_t>(out) & 7) == 0,
                 Status::kInvalidArgument, "attention: misaligned operands");

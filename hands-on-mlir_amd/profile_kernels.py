@@ -6,6 +6,7 @@ what:  gemm1      FFN1 GEMM + bias + tanh-GELU, M=1024 K=768 N=3072 (tuned kerne
        gemm5      BERT-large FFN2 GEMM, M=16384 K=4096 N=1024
        layernorm  in-place layer norm, 16384 x 1024
        attention  packed-QKV attention, b8 s128 h12
+       attention5 packed-QKV attention, b32 s512 h16, full-length sequences
        lnpair     the layer-norm pair at BERT-large size: GEMM + row statistics
                   16384x1024x1024, then the GEMM of the normalised rows
                   16384x4096x1024, next to the two plain GEMMs
@@ -41,6 +42,9 @@ def main():
     elif what == "attention":
         lens = (ctypes.c_int32 * 8)(83, 128, 57, 101, 32, 120, 64, 99)
         print(f"attention b8 s128 h12: {drv.homTimeAttention(8, 128, 12, lens, iters, 3) * 1e3:.2f} us")
+    elif what == "attention5":
+        lens = (ctypes.c_int32 * 32)(*([512] * 32))
+        print(f"attention b32 s512 h16: {drv.homTimeAttention(32, 512, 16, lens, iters, 3) * 1e3:.2f} us")
     elif what == "lnpair":
         import torch
         M = rt.MemRef.from_tensor
