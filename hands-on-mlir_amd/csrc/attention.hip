@@ -67,7 +67,7 @@ __device__ __forceinline__ float pairSum(float v) {
 
 template <int NW>
 __global__ __launch_bounds__(NW *kWave)
-__attribute__((amdgpu_waves_per_eu(2, 3))) void bertAttentionKernel(
+__attribute__((amdgpu_waves_per_eu(2, NW == 4 ? 4 : 2))) void bertAttentionKernel(
     const _Float16 *__restrict__ qkv, const int32_t *__restrict__ cu,
     _Float16 *__restrict__ out, int seq, int heads, float scale) {
   constexpr int kThreads = NW * kWave;
