@@ -145,6 +145,11 @@ def main():
     at_ms = drv.homTimeAttention(8, 128, 12, lens, 2000, 50)
     kernels["attention_b8_s128_h12"] = {"us": at_ms * 1e3, "GB/s": gbs(6291492, at_ms),
                                         "dense_TFLOP/s": 402653184 / (at_ms * 1e-3) / 1e12}
+    full = (ctypes.c_int32 * 32)(*([512] * 32))
+    at5_ms = drv.homTimeAttention(32, 512, 16, full, 200, 10)
+    kernels["attention_b32_s512_h16_full_length"] = {
+        "us": at5_ms * 1e3, "GB/s": gbs(2 * (32 * 512 * 3072 + 32 * 512 * 1024) + 4 * 33, at5_ms),
+        "dense_TFLOP/s": 4.0 * 32 * 16 * 512 * 512 * 64 / (at5_ms * 1e-3) / 1e12}
     for (m, n, k, act, tag) in [(16384, 4096, 1024, 1, "gemm_gelu_16384x4096x1024"),
                                 (16384, 1024, 4096, 0, "gemm_16384x1024x4096"),
                                 (64, 1024, 4096, 0, "gemm_skinny_64x1024x4096"),

@@ -69,15 +69,34 @@ template <int NW>
 __global__ __launch_bounds__(NW *kWave)
 __attribute__((amdgpu_waves_per_eu(2, NW == 4 ? 4 : 2))) void bertAttentionKernel(
     const _Float16 *__restrict__ qkv, const int32_t *__restrict__ cu,
-    _Float16 *__restrict__ out, int seq, int heads, float scale) {
+    _Float16 *__restrict__ out, int seq, int heads, int numQTiles, int pairs,
+    float scale) {
   constexpr int kThreads = NW * kWave;
   __shared__ __attribute__((aligned(16))) unsigned char sK[kTileBytes];
   __shared__ __attribute__((aligned(16))) unsigned char sV[kTileBytes];
 
   const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
   const int l32 = lane % 32, hb = lane / 32;
-  const int head = blockIdx.y, b = blockIdx.z;
-  const int q0 = blockIdx.x * (NW * 32) + wave * 32;
+  // Workgroup id -> (query tile, head, batch).  Workgroups are dealt to the 8
+  // XCDs round-robin by id, and the query tiles of one (batch, head) read the
+  // same K and V: ids that differ by 8 (same XCD, launched back to back) walk
+  // the query tiles of one pair, so K/V are fetched into one L2 once instead
+  // of once per XCD.  Needs the pair count to be a multiple of 8; the
+  // 2-wavefront variant (few workgroups, launch-bound) keeps the plain order.
+  int qTile, pair;
+  {
+    const int id = blockIdx.x;
+    if (NW == 4 && pairs % 8 == 0) {
+      const int t = id / 8;
+      qTile = t % numQTiles;
+      pair = (t / numQTiles) * 8 + id % 8;
+    } else {
+      qTile = id % numQTiles;
+      pair = id / numQTiles;
+    }
+  }
+  const int head = pair % heads, b = pair / heads;
+  const int q0 = qTile * (NW * 32) + wave * 32;
   const int cuLo = cu[b], cuHi = cu[b + 1]; // consumed after the first loads are out
 
   const int64_t tokStride = int64_t(3) * heads * kHeadDim;
@@ -129,7 +148,7 @@ __attribute__((amdgpu_waves_per_eu(2, NW == 4 ? 4 : 2))) void bertAttentionKerne
   int len = cuHi - cuLo;
   len = len < 0 ? 0 : (len > seq ? seq : len);
   // A workgroup whose query rows are all padding has nothing to compute.
-  if (int(blockIdx.x) * (NW * 32) >= len) {
+  if (qTile * (NW * 32) >= len) {
     const int q = q0 + l32;
     if (q < seq) {
       half4 z;
@@ -396,16 +415,16 @@ Status launchBertAttentionF16(const _Float16 *qkv, const int32_t *cuSeqlens,
   bool wide = pairs * ((seq + 127) / 128) >= int64_t(cus) || seq <= 32;
   if (const char *force = getenv("HOM_ATTENTION_WAVES")) // profiling knob: 2 or 4
     wide = atoi(force) == 4;
+  HOM_CHECK_RET(pairs * ((seq + 63) / 64) < (int64_t(1) << 31),
+                Status::kInvalidArgument, "attention: too many workgroups");
   if (wide) {
-    dim3 grid((unsigned)((seq + 127) / 128), (unsigned)heads, (unsigned)bs);
-    bertAttentionKernel<4><<<grid, dim3(256), 0, s>>>(qkv, cuSeqlens, out,
-                                                      int(seq), int(heads),
-                                                      scale);
+    const int nq = int((seq + 127) / 128);
+    bertAttentionKernel<4><<<dim3((unsigned)(nq * pairs)), dim3(256), 0, s>>>(
+        qkv, cuSeqlens, out, int(seq), int(heads), nq, int(pairs), scale);
   } else {
-    dim3 grid((unsigned)((seq + 63) / 64), (unsigned)heads, (unsigned)bs);
-    bertAttentionKernel<2><<<grid, dim3(128), 0, s>>>(qkv, cuSeqlens, out,
-                                                      int(seq), int(heads),
-                                                      scale);
+    const int nq = int((seq + 63) / 64);
+    bertAttentionKernel<2><<<dim3((unsigned)(nq * pairs)), dim3(128), 0, s>>>(
+        qkv, cuSeqlens, out, int(seq), int(heads), nq, int(pairs), scale);
   }
   HOM_HIP_RET(hipGetLastError(), Status::kInternal);
   return Status::kSuccess;
