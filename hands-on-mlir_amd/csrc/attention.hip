@@ -115,8 +115,8 @@ __attribute__((amdgpu_waves_per_eu(2, NW == 4 ? 4 : 2))) void bertAttentionKerne
   // length has arrived, and the next chunk's loads fly while this one is
   // multiplied.  The 4-wavefront variant serves long sequences with many
   // workgroups per CU, which cover each other's staging; there the early loads
-  // are wasted on all-padding workgroups and the plain copy loop measured 3-8 %
-  // faster.
+  // are wasted on all-padding workgroups, and prefetching the next chunk into
+  // registers measured 4-8 % slower than loading each chunk when it is due.
   constexpr bool kPrefetch = NW == 2;
   constexpr int VPT = kChunk * 8 / kThreads; // vectors of K (and of V) per thread
   half8 rk[VPT], rv[VPT];
