@@ -25,6 +25,7 @@
 // ds_read_b64_tr_b16 (the transposing LDS read) from the row-major V tile.
 // LDS rows are 128 bytes, unpadded; 16-byte chunks (K) / 64-byte groups (V) are
 // XOR-permuted by row so that the fragment reads are bank-conflict free.
+#include "cross_lane.h"
 #include "kernels.h"
 
 namespace hom {
@@ -48,21 +49,6 @@ __device__ __forceinline__ int swzK(int row, int chunk) {
 // 64-byte group g of V row k lives at position g ^ ((k >> 1) & 1)
 __device__ __forceinline__ int swzV(int k, int group) {
   return group ^ ((k >> 1) & 1);
-}
-
-// Combine a value with the one in lane ^ 32.  v_permlane32_swap exchanges the
-// upper half of its first operand with the lower half of its second; given
-// the same value twice it returns (lower-half values, upper-half values) in
-// every lane pair -- one VALU instruction where a shuffle is an LDS round trip.
-__device__ __forceinline__ float pairMax(float v) {
-  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v),
-                                                  __float_as_uint(v), false, false);
-  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
-}
-__device__ __forceinline__ float pairSum(float v) {
-  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v),
-                                                  __float_as_uint(v), false, false);
-  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
 template <int NW>

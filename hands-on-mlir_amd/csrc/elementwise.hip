@@ -7,6 +7,7 @@
 //   gather       include/NVGPUKernels/GatherRunner.h:32-77
 //   cu_seqlens   include/NVGPUKernels/CuSeqLen.h:28-74
 //   row stats    include/NVGPUKernels/Layernorm.h:33-195 (ApplyFinalReduction)
+#include "cross_lane.h"
 #include "kernels.h"
 
 namespace hom {
@@ -220,11 +221,8 @@ __global__ __launch_bounds__(256) void rowStatsKernel(
     s += x;
     sq += x * x;
   }
-#pragma unroll
-  for (int off = kWave / 2; off > 0; off >>= 1) {
-    s += __shfl_xor(s, off, kWave);
-    sq += __shfl_xor(sq, off, kWave);
-  }
+  s = waveSum(s);
+  sq = waveSum(sq);
   if (lane == 0) {
     const float m = s / float(n);
     const float ms = sq / float(n);

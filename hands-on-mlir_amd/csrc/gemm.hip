@@ -41,6 +41,7 @@
 //  * "staged" kernels (any shape / alignment, and the first bring-up path):
 //    global -> registers -> LDS with two LDS buffers and 32-wide slabs; row-major
 //    B is interleaved into (k, k+1) half2 pairs while it is staged.
+#include "cross_lane.h"
 #include "kernels.h"
 
 #include <algorithm>
@@ -133,25 +134,6 @@ template <int EPI> __device__ __forceinline__ float activate(float v) {
     return geluErf(v);
   if (EPI == int(Epilogue::kGeluTanh))
     return geluTanh(v);
-  return v;
-}
-
-// Sum over groups of N consecutive lanes (N = 4, 8 or 16, groups aligned to
-// N) with data-parallel-primitive adds: quad permutes exchange lanes ^1 and ^2,
-// the half-row and row mirrors pair each lane with one of the other quad /
-// the other half of its 16-lane row.  No LDS round trips, unlike shuffles.
-template <int CTRL> __device__ __forceinline__ float addDpp(float v) {
-  return v + __int_as_float(__builtin_amdgcn_update_dpp(
-                 0, __float_as_int(v), CTRL, 0xf, 0xf, false));
-}
-template <int N> __device__ __forceinline__ float sumAcrossLanes(float v) {
-  static_assert(N == 4 || N == 8 || N == 16, "group size");
-  v = addDpp<0xB1>(v); // quad_perm [1,0,3,2]
-  v = addDpp<0x4E>(v); // quad_perm [2,3,0,1]
-  if (N >= 8)
-    v = addDpp<0x141>(v); // row_half_mirror
-  if (N >= 16)
-    v = addDpp<0x140>(v); // row_mirror
   return v;
 }
 
@@ -1391,10 +1373,8 @@ __global__ __launch_bounds__(256) void rowStatsFinalizeKernel(
       sq += v[u][1];
     }
   }
-  s += __shfl_xor(s, 16, kWave);
-  sq += __shfl_xor(sq, 16, kWave);
-  s += __shfl_xor(s, 32, kWave);
-  sq += __shfl_xor(sq, 32, kWave);
+  s = pairSum(rowPairSum(s));
+  sq = pairSum(rowPairSum(sq));
   if (q == 0 && m < M) {
     const float mu = s / float(N);
     const float rstd = 1.0f / sqrtf(sq / float(N) - mu * mu + eps);

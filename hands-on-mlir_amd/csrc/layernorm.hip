@@ -7,9 +7,10 @@
 //
 // The kernel is bandwidth bound: each row is read once with 128-bit loads and
 // stays in registers for the two statistic passes; one 64-lane wavefront owns
-// a row and reduces with cross-lane shuffles (no LDS).  Rows that do not fit
+// a row and reduces across lanes inside the vector ALU (no LDS).  Rows that do not fit
 // that scheme (odd lengths, very long rows) take a workgroup-per-row kernel
 // that reduces through LDS.
+#include "cross_lane.h"
 #include "kernels.h"
 
 namespace hom {
@@ -26,13 +27,6 @@ template <> struct Vec16<float> {
   static constexpr int kN = 4;
   typedef float type __attribute__((ext_vector_type(4)));
 };
-
-__device__ __forceinline__ float waveSum(float v) {
-#pragma unroll
-  for (int off = kWave / 2; off > 0; off >>= 1)
-    v += __shfl_xor(v, off, kWave);
-  return v;
-}
 
 // One wavefront per row; VPL 16-byte vectors per lane.
 template <typename T, int VPL, bool HAS_RES, bool HAS_AFFINE>
