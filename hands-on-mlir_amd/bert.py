@@ -66,6 +66,12 @@ class BertEncoder:
         assert ms > 0, "timing failed"
         return ms
 
+    def set_gemm_choice(self, role, gemm_num, split_k=1):
+        """Pin the manifest kernel (1-based) of one GEMM role ("qkv", "out", "ffn1", "ffn2")."""
+        idx = ("qkv", "out", "ffn1", "ffn2").index(role)
+        if self.drv.homBertSetGemmChoice(self.h, idx, gemm_num, split_k) != 0:
+            raise ValueError(f"bad kernel choice {gemm_num}/{split_k} for {role}")
+
     def gemm_choices(self):
         buf = (ctypes.c_int32 * 8)()
         self.drv.homBertGetGemmChoices(self.h, buf)

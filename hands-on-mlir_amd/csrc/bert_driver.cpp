@@ -388,6 +388,22 @@ DRV_EXPORT void homBertGetGemmChoices(HomBertEncoder *e, int32_t *out8) {
   }
 }
 
+// Pins the manifest kernel (1-based, as cutlassGemmF16 takes it) and split-K
+// factor of one GEMM role: 0 QKV, 1 output projection, 2 FFN1, 3 FFN2.  What a
+// compiled module carries as constants; here it lets the autotuner time
+// candidates inside the encoder graph, where operands arrive cold from the
+// previous kernel.  A captured graph must be captured again afterwards.
+DRV_EXPORT int homBertSetGemmChoice(HomBertEncoder *e, int role,
+                                    int32_t gemmNum, int32_t splitK) {
+  GemmChoice *c[4] = {&e->cQkv, &e->cOut, &e->cFfn1, &e->cFfn2};
+  if (role < 0 || role > 3 || gemmNum < 1 || gemmNum > homGemmManifestSize() ||
+      splitK < 1)
+    return -1;
+  c[role]->gemmNum = gemmNum;
+  c[role]->splitK = splitK;
+  return 0;
+}
+
 // ---- single-operator timing through the boundary -------------------------
 // Each helper enqueues `iters` back-to-back calls of one entry point between
 // two events on a private stream and returns mean milliseconds per call.
