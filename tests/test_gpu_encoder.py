@@ -73,6 +73,32 @@ def test_small_encoder_eager_and_graph(gpu, oracle, synth, gemm_mode, gelu):
         enc.close()
 
 
+def test_pinned_gemm_kernels_in_the_graph(gpu, rt, oracle, synth):
+    """The autotuner's in-graph pass pins one GEMM role at a time to another manifest kernel and
+    captures again: every such graph must still compute the encoder."""
+    bert = importlib.import_module("hands-on-mlir_amd.bert")
+    model = synth.bert_encoder(layers=2, hidden=128, heads=2, ffn=512, bs=3, seq=64, vocab=1000, config=40)
+    number = {n: i + 1 for i, n, _, _ in rt.manifest()}
+    want32 = oracle_forward(oracle, model, "erf")
+    enc = bert.BertEncoder(2, 128, 2, 512, 3, 64, 1000, gemm_mode=1, gelu_form="erf")
+    try:
+        enc.load(model)
+        enc.set_inputs(ids=model["ids"], mask=model["mask"])
+        tile = "hom_gfx950_mfma_f16_s32x32x16gemm_f16_128x64_64x2r2_w2x2_nn_align8_"
+        for role, epi, split in (("qkv", "linear", 1), ("out", "linear", 2), ("ffn1", "gelu", 1), ("ffn2", "linear", 3)):
+            enc.set_gemm_choice(role, number[tile + epi], split)
+            assert enc.gemm_choices()[role] == (number[tile + epi], split)
+            enc.capture()
+            enc.replay()
+            check(enc.output(), want32, model["lens"], f"{role} pinned to 128x64, split-K {split}")
+        with pytest.raises(ValueError):
+            enc.set_gemm_choice("out", 0, 1)
+        with pytest.raises(ValueError):
+            enc.set_gemm_choice("out", 1, 0)
+    finally:
+        enc.close()
+
+
 def test_bert_base_b8_s128(gpu, oracle, synth):
     bert = importlib.import_module("hands-on-mlir_amd.bert")
     model = synth.bert_encoder()
