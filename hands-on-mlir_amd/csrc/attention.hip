@@ -102,7 +102,8 @@ __attribute__((amdgpu_waves_per_eu(2, NW == 4 ? 4 : 2))) void bertAttentionKerne
   // multiplied.  The 4-wavefront variant serves long sequences with many
   // workgroups per CU, which cover each other's staging; there the early loads
   // are wasted on all-padding workgroups, and prefetching the next chunk into
-  // registers measured 4-8 % slower than loading each chunk when it is due.
+  // registers measured 3-8 % slower than loading each chunk when it is due
+  // (also with barriers that do not wait for the prefetch).
   constexpr bool kPrefetch = NW == 2;
   constexpr int VPT = kChunk * 8 / kThreads; // vectors of K (and of V) per thread
   half8 rk[VPT], rv[VPT];
