@@ -9,10 +9,14 @@
 // Replaces the cuDNN fused attention reached through
 // include/NVGPUKernels/BertAttentionRunner.h:113-136.
 //
-// A workgroup of NW wavefronts handles 32*NW query rows of one (batch, head);
-// each wavefront owns 32 of them.  Keys are walked in chunks of 128: the whole
-// workgroup stages the chunk's K and V rows into LDS (one barrier), then every
-// wavefront runs over it in blocks of 64 keys without further synchronisation.
+// A workgroup of four wavefronts handles 128 or 64 query rows of one (batch,
+// head): each wavefront owns 32 rows and walks every key block (long
+// sequences, many workgroups), or two wavefronts share 32 rows and take every
+// other key block (short sequences: fewer workgroups than CUs, the key walk of
+// one wavefront is the critical path; the two halves are merged through LDS).
+// Keys are walked in chunks of 128: the whole workgroup stages the chunk's K
+// and V rows into LDS (one barrier), then the wavefronts run over it in blocks
+// of 64 keys without further synchronisation.
 // Both contractions run on v_mfma_f32_32x32x16_f16 and are issued transposed:
 //   S^T = K Q^T   (A operand = K rows from LDS, B operand = Q rows in registers)
 //   O^T = V^T P^T (A operand = V columns, B operand = P rows)
@@ -27,6 +31,8 @@
 // XOR-permuted by row so that the fragment reads are bank-conflict free.
 #include "cross_lane.h"
 #include "kernels.h"
+
+#include <cstring>
 
 namespace hom {
 namespace {
@@ -51,18 +57,25 @@ __device__ __forceinline__ int swzV(int k, int group) {
   return group ^ ((k >> 1) & 1);
 }
 
-template <int NW>
+// NW wavefronts per workgroup, KS of them share each group of 32 query rows
+// and split its key blocks between them (KS = 1: every wavefront walks all
+// keys of its own 32 rows; KS = 2: half the serial work per wavefront, for
+// short sequences where there are fewer workgroups than CUs and the key walk
+// of one wavefront is the critical path; the halves are merged through LDS).
+template <int NW, int KS>
 __global__ __launch_bounds__(NW *kWave)
-__attribute__((amdgpu_waves_per_eu(2, NW == 4 ? 4 : 2))) void bertAttentionKernel(
+__attribute__((amdgpu_waves_per_eu(2, KS == 1 ? 4 : 2))) void bertAttentionKernel(
     const _Float16 *__restrict__ qkv, const int32_t *__restrict__ cu,
     _Float16 *__restrict__ out, int seq, int heads, int numQTiles, int pairs,
     float scale) {
   constexpr int kThreads = NW * kWave;
-  __shared__ __attribute__((aligned(16))) unsigned char sK[kTileBytes];
-  __shared__ __attribute__((aligned(16))) unsigned char sV[kTileBytes];
+  constexpr int QG = NW / KS; // groups of 32 query rows per workgroup
+  __shared__ __attribute__((aligned(16))) unsigned char smem[2 * kTileBytes];
+  unsigned char *const sK = smem, *const sV = smem + kTileBytes;
 
   const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
   const int l32 = lane % 32, hb = lane / 32;
+  const int qg = wave % QG, kh = wave / QG; // query group, key share
   // Workgroup id -> (query tile, head, batch).  Workgroups are dealt to the 8
   // XCDs round-robin by id, and the query tiles of one (batch, head) read the
   // same K and V: ids that differ by 8 (same XCD, launched back to back) walk
@@ -72,7 +85,7 @@ __attribute__((amdgpu_waves_per_eu(2, NW == 4 ? 4 : 2))) void bertAttentionKerne
   int qTile, pair;
   {
     const int id = blockIdx.x;
-    if (NW == 4 && pairs % 8 == 0) {
+    if (KS == 1 && pairs % 8 == 0) {
       const int t = id / 8;
       qTile = t % numQTiles;
       pair = (t / numQTiles) * 8 + id % 8;
@@ -82,7 +95,7 @@ __attribute__((amdgpu_waves_per_eu(2, NW == 4 ? 4 : 2))) void bertAttentionKerne
     }
   }
   const int head = pair % heads, b = pair / heads;
-  const int q0 = qTile * (NW * 32) + wave * 32;
+  const int q0 = qTile * (QG * 32) + qg * 32;
   const int cuLo = cu[b], cuHi = cu[b + 1]; // consumed after the first loads are out
 
   const int64_t tokStride = int64_t(3) * heads * kHeadDim;
@@ -93,18 +106,17 @@ __attribute__((amdgpu_waves_per_eu(2, NW == 4 ? 4 : 2))) void bertAttentionKerne
   const int64_t outStride = int64_t(heads) * kHeadDim;
   _Float16 *oBase = out + int64_t(b) * seq * outStride + head * kHeadDim;
 
-  // 2-wavefront variant (short sequences, few workgroups: latency is what
+  // Key-split variant (short sequences, few workgroups: latency is what
   // counts): K and V rows of a 128-key chunk travel global -> registers -> LDS,
   // 16 bytes per vector.  The loads are unconditional (rows past the end of the tensor
   // are clamped, rows past the sequence end are zeroed on the way to LDS), so
   // the first chunk's loads and the Q loads are issued before the sequence
-  // length has arrived, and the next chunk's loads fly while this one is
-  // multiplied.  The 4-wavefront variant serves long sequences with many
+  // length has arrived.  The other variant serves long sequences with many
   // workgroups per CU, which cover each other's staging; there the early loads
   // are wasted on all-padding workgroups, and prefetching the next chunk into
   // registers measured 3-8 % slower than loading each chunk when it is due
   // (also with barriers that do not wait for the prefetch).
-  constexpr bool kPrefetch = NW == 2;
+  constexpr bool kPrefetch = KS == 2;
   constexpr int VPT = kChunk * 8 / kThreads; // vectors of K (and of V) per thread
   half8 rk[VPT], rv[VPT];
   auto loadChunk = [&](int key0) {
@@ -135,9 +147,9 @@ __attribute__((amdgpu_waves_per_eu(2, NW == 4 ? 4 : 2))) void bertAttentionKerne
   int len = cuHi - cuLo;
   len = len < 0 ? 0 : (len > seq ? seq : len);
   // A workgroup whose query rows are all padding has nothing to compute.
-  if (qTile * (NW * 32) >= len) {
+  if (qTile * (QG * 32) >= len) {
     const int q = q0 + l32;
-    if (q < seq) {
+    if (q < seq && kh == 0) {
       half4 z;
 #pragma unroll
       for (int e = 0; e < 4; e++)
@@ -232,7 +244,7 @@ __attribute__((amdgpu_waves_per_eu(2, NW == 4 ? 4 : 2))) void bertAttentionKerne
       loadChunk(key0 + kChunk);
     __syncthreads();
 
-    for (int blk = 0; blk < live; blk += 64) {
+    for (int blk = kh * 64; blk < live; blk += 64 * KS) {
       // ---- S^T = K Q^T for two 32-key sub-blocks ----
       // All eight K fragments are requested before the first MFMA: read one
       // at a time, each MFMA would wait out a full LDS round trip.
@@ -351,6 +363,41 @@ __attribute__((amdgpu_waves_per_eu(2, NW == 4 ? 4 : 2))) void bertAttentionKerne
     }
   }
 
+  // ---- merge the key shares ----
+  // Share 1 hands (reference, sum, O) of its rows to share 0 through LDS, in
+  // the layout [query group][value][lane]; lanes of the two wavefronts hold
+  // the same (row, columns).  With references m0, m1 in raw score units and
+  // m = max(m0, m1): O = O0 2^((m0-m)c) + O1 2^((m1-m)c), the same for the
+  // sums.  A share that saw no valid key has m1 = -inf and weight 0; share 0
+  // always owns the first block, which has one.
+  if constexpr (KS == 2) {
+    static_assert(QG * 34 * kWave * 4 <= 2 * kTileBytes, "exchange fits the K/V tiles");
+    float *xch = reinterpret_cast<float *>(smem) + qg * (34 * kWave) + lane;
+    __syncthreads(); // every wavefront is done with K and V
+    if (kh == 1) {
+#pragma unroll
+      for (int d = 0; d < 2; d++)
+#pragma unroll
+        for (int e = 0; e < 16; e++)
+          xch[(d * 16 + e) * kWave] = accO[d][e];
+      xch[32 * kWave] = rowMax;
+      xch[33 * kWave] = rowSum;
+    }
+    __syncthreads();
+    if (kh == 1)
+      return;
+    const float m1 = xch[32 * kWave], l1 = xch[33 * kWave];
+    const float m = fmaxf(rowMax, m1);
+    const float c0 = __builtin_amdgcn_exp2f((rowMax - m) * scaleLog2e);
+    const float c1 = __builtin_amdgcn_exp2f((m1 - m) * scaleLog2e);
+    rowSum = rowSum * c0 + l1 * c1;
+#pragma unroll
+    for (int d = 0; d < 2; d++)
+#pragma unroll
+      for (int e = 0; e < 16; e++)
+        accO[d][e] = accO[d][e] * c0 + xch[(d * 16 + e) * kWave] * c1;
+  }
+
   // ---- normalise and store ----
   // accO[d][e]: column dcol = d*32 + 8*(e/4) + 4*hb + e%4 of query row l32.
   const int q = q0 + l32;
@@ -395,22 +442,24 @@ Status launchBertAttentionF16(const _Float16 *qkv, const int32_t *cuSeqlens,
                 Status::kInvalidArgument, "attention: misaligned operands");
   if (bs == 0 || seq == 0 || heads == 0)
     return Status::kSuccess;
-  // 128 query rows per workgroup when that still gives every CU work,
-  // otherwise 64 (K/V of a (batch, head) are then staged by two workgroups).
+  // 128 query rows per workgroup (one wavefront per 32 rows) when that still
+  // gives every CU work, otherwise 64 with the keys split over two wavefronts
+  // per 32 rows (K/V of a (batch, head) are then staged by two workgroups).
   const int cus = deviceInfo().computeUnits;
   const int64_t pairs = bs * heads;
   bool wide = pairs * ((seq + 127) / 128) >= int64_t(cus) || seq <= 32;
-  if (const char *force = getenv("HOM_ATTENTION_WAVES")) // profiling knob: 2 or 4
-    wide = atoi(force) == 4;
+  // profiling knob: HOM_ATTENTION_VARIANT=wide | split
+  if (const char *force = getenv("HOM_ATTENTION_VARIANT"))
+    wide = strcmp(force, "wide") == 0;
   HOM_CHECK_RET(pairs * ((seq + 63) / 64) < (int64_t(1) << 31),
                 Status::kInvalidArgument, "attention: too many workgroups");
   if (wide) {
     const int nq = int((seq + 127) / 128);
-    bertAttentionKernel<4><<<dim3((unsigned)(nq * pairs)), dim3(256), 0, s>>>(
+    bertAttentionKernel<4, 1><<<dim3((unsigned)(nq * pairs)), dim3(256), 0, s>>>(
         qkv, cuSeqlens, out, int(seq), int(heads), nq, int(pairs), scale);
   } else {
     const int nq = int((seq + 63) / 64);
-    bertAttentionKernel<2><<<dim3((unsigned)(nq * pairs)), dim3(128), 0, s>>>(
+    bertAttentionKernel<4, 2><<<dim3((unsigned)(nq * pairs)), dim3(256), 0, s>>>(
         qkv, cuSeqlens, out, int(seq), int(heads), nq, int(pairs), scale);
   }
   HOM_HIP_RET(hipGetLastError(), Status::kInternal);
