@@ -1,0 +1,41 @@
+// The part of the reference's autotune pass that touches the kernel library
+// (lib/Dialect/HOMNVGPU/HOMNVGPUAutotunePass.cpp:52-92), without the MLIR
+// types around it: same include, same namespace, same calls.  Built by
+// tests/test_abi.py against include/NVGPUKernels/GemmProfiler.h and
+// libhom_amdgpu_runner_utils.so; with "run" as its argument it profiles one
+// shape on the GPU and prints the result.
+#include "NVGPUKernels/GemmProfiler.h"
+
+#include <cstdio>
+#include <cstring>
+
+namespace {
+struct MatmulOpStandIn {
+  int64_t kernelName = 0;
+  int32_t splitK = 0;
+  void setKernelName(int64_t v) { kernelName = v; }
+  void setSplitKFactor(int32_t v) { splitK = v; }
+};
+
+void profileMatmulImpl(MatmulOpStandIn &gemm, int64_t M, int64_t N, int64_t K,
+                       int64_t act, float alpha, float beta) {
+  using namespace mlir::hands_on_mlir::homnvgpu_kernel;
+  static GemmProfiler profiler(M, N, K, act, alpha, beta);
+  auto [bestIdx, bestSplitKFactor] = profiler.profile(M, N, K, act, alpha, beta);
+  gemm.setKernelName(bestIdx + 1);
+  gemm.setSplitKFactor(bestSplitKFactor);
+}
+} // namespace
+
+int main(int argc, char **argv) {
+  if (argc > 1 && strcmp(argv[1], "run") == 0) {
+    MatmulOpStandIn op;
+    profileMatmulImpl(op, 256, 768, 768, 0, 1.0f, 0.0f);
+    printf("%lld %d %s\n", (long long)op.kernelName, op.splitK,
+           op.kernelName >= 1 ? homGemmManifestName(int32_t(op.kernelName - 1))
+                              : "none");
+    return op.kernelName >= 1 && op.splitK >= 1 ? 0 : 1;
+  }
+  printf("%d\n", homGemmManifestSize());
+  return 0;
+}

@@ -118,6 +118,37 @@ print(json.dumps(out))
     assert "_64x2r" in picks["1024x30522x768x0"][0] and picks["1024x30522x768x0"][1] == 1  # even N: pipe family
 
 
+def build_autotune_usage(tmp_path):
+    exe = str(tmp_path / "autotune_pass_usage")
+    lib_dir = os.path.join(ROOT, "hands-on-mlir_amd", "lib")
+    cmd = ["g++", "-std=c++17", "-O1", "-Wall", "-I", os.path.join(ROOT, "include"),
+           os.path.join(ROOT, "tests", "modules", "autotune_pass_usage.cpp"),
+           "-L", lib_dir, "-lhom_amdgpu_runner_utils", f"-Wl,-rpath,{lib_dir}", "-o", exe]
+    res = subprocess.run(cmd, capture_output=True, text=True, timeout=300)
+    assert res.returncode == 0, res.stderr
+    return exe
+
+
+def test_autotune_pass_source_compiles_against_the_profiler_header(rt, tmp_path):
+    """The reference's pass includes NVGPUKernels/GemmProfiler.h and calls GemmProfiler::profile;
+    its library-facing code must compile and link unchanged against this repo's header and library."""
+    rt.load_runtime()
+    exe = build_autotune_usage(tmp_path)
+    res = subprocess.run([exe], capture_output=True, text=True, timeout=60)
+    assert res.returncode == 0, res.stderr
+    assert int(res.stdout.strip()) == len(rt.manifest())
+
+
+@pytest.mark.gpu
+def test_autotune_pass_usage_runs_on_the_gpu(rt, tmp_path):
+    rt.load_runtime()
+    exe = build_autotune_usage(tmp_path)
+    res = subprocess.run([exe, "run"], capture_output=True, text=True, timeout=300)
+    assert res.returncode == 0, res.stdout + res.stderr
+    num, split, name = res.stdout.strip().splitlines()[-1].split()
+    assert 1 <= int(num) <= len(rt.manifest()) and int(split) >= 1 and name.endswith("_linear")
+
+
 # ---- argument checking: runs without a GPU because every check precedes the
 # first HIP call.  Default mode aborts (reference: assert / exit(1)); mode 1
 # records the message instead.
