@@ -9,13 +9,17 @@ from . import hom_runtime as rt
 
 
 class BertEncoder:
-    def __init__(self, layers, hidden, heads, ffn, bs, seq, vocab, gemm_mode=1, gelu_form="erf"):
+    def __init__(self, layers, hidden, heads, ffn, bs, seq, vocab, gemm_mode=1, gelu_form="erf",
+                 lm_head=False):
         self.drv = rt.load_driver()
         self.dims = dict(layers=layers, hidden=hidden, heads=heads, ffn=ffn, bs=bs, seq=seq, vocab=vocab)
         self.gemm_mode = gemm_mode
         self.h = self.drv.homBertCreate(layers, hidden, heads, ffn, bs, seq, vocab, gemm_mode,
                                         1 if gelu_form == "tanh" else 0)
         assert self.h, "homBertCreate failed"
+        self.lm_head = lm_head
+        if lm_head:
+            assert self.drv.homBertEnableLmHead(self.h) == 0, "homBertEnableLmHead failed"
 
     def close(self):
         if self.h:
@@ -37,6 +41,11 @@ class BertEncoder:
                 self._upload(l, which, tr(w[key]))
         self._upload(0, 4, model["word"])
         self._upload(0, 5, model["pos_type"])
+        if self.lm_head:
+            # the decoder is tied to the word embeddings (BertForMaskedLM): logits = t . word^T, so the
+            # [K, N] operand of the manifest path is word^T and the [N, K] operand of the nvte path is word
+            self._upload(0, 6, tr(model["w_transform"]))
+            self._upload(0, 7, model["word"] if self.gemm_mode == 0 else model["word"].T)
 
     def set_inputs(self, ids=None, mask=None, hidden=None):
         p = lambda a, dt: (np.ascontiguousarray(a, dt).ctypes.data_as(ctypes.c_void_p)
@@ -59,6 +68,12 @@ class BertEncoder:
         d = self.dims
         out = np.empty((d["bs"], d["seq"], d["hidden"]), np.float16)
         assert self.drv.homBertGetOutput(self.h, out.ctypes.data_as(ctypes.c_void_p)) == 0
+        return out
+
+    def logits(self):
+        d = self.dims
+        out = np.empty((d["bs"], d["seq"], d["vocab"]), np.float16)
+        assert self.drv.homBertGetLogits(self.h, out.ctypes.data_as(ctypes.c_void_p)) == 0
         return out
 
     def time(self, steps, warmup, graph=True, from_ids=True):

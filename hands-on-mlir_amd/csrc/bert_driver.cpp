@@ -11,7 +11,10 @@
 //            cu_seqlens; gather + add + layernorm (embeddings);
 //            per layer: QKV GEMM, attention, out-proj GEMM (+residual, in
 //            place), layernorm, FFN1 GEMM+GELU, FFN2 GEMM (+residual, in
-//            place), layernorm.
+//            place), layernorm;
+//            optionally the masked-LM head of the reference's BertForMaskedLM
+//            graph (examples/torch/bert/bert.cu:25,140-163: logits
+//            [b, s, vocab]): dense + GELU, layernorm, vocabulary projection.
 // Because that list is static, the driver can also capture it once into a HIP
 // graph and replay it, which removes the per-call launch overhead that
 // dominates at batch 8 x seq 128.
@@ -67,7 +70,12 @@ struct HomBertEncoder {
   Tensor mask;      // int64 [b, s]
   Tensor cu;        // int32 [b+1]
   Tensor h, emb, qkv, attn, f;
-  GemmChoice cQkv, cOut, cFfn1, cFfn2;
+  // masked-LM head (homBertEnableLmHead): transform weight [1,H,H], decoder
+  // weight [1,H,V] ([1,H,H] / [1,V,H] on the nvte path), transform output and
+  // logits
+  bool lmHead = false;
+  Tensor wTransform, wDecoder, t, logits;
+  GemmChoice cQkv, cOut, cFfn1, cFfn2, cTransform, cDecoder;
   hipStream_t stream = nullptr;
   hipGraph_t graph = nullptr;
   hipGraphExec_t graphExec = nullptr;
@@ -157,6 +165,13 @@ void callList(HomBertEncoder *e, int fromIds) {
     gemm(e, e->f, w.w2, e->h, e->h, 0, 1.0f, e->cFfn2);
     nvteLayernormF16(e->h.m.rank, e->h.m.descriptor, e->eps);
   }
+  if (e->lmHead) {
+    // BertLMPredictionHead with default-initialised (folded away) biases and
+    // affine parameters: t = LN(GELU(h Wt)); logits = t Wd
+    gemm(e, e->h, e->wTransform, e->t, e->t, geluAct, 0.0f, e->cTransform);
+    nvteLayernormF16(e->t.m.rank, e->t.m.descriptor, e->eps);
+    gemm(e, e->t, e->wDecoder, e->logits, e->logits, 0, 0.0f, e->cDecoder);
+  }
 }
 
 } // namespace
@@ -213,6 +228,32 @@ DRV_EXPORT HomBertEncoder *homBertCreate(int layers, int hidden, int heads,
   return e;
 }
 
+// Adds the masked-LM head to the call list: allocates its two weights
+// (upload with which = 6 transform [H,H], 7 decoder [H,V]; [N,K] layouts when
+// gemmMode == 0), the transform buffer and the logits [b, s, vocab].  A graph
+// captured before this call must be captured again.
+DRV_EXPORT int homBertEnableLmHead(HomBertEncoder *e) {
+  if (e->lmHead)
+    return 0;
+  const bool nk = e->gemmMode == 0;
+  e->wTransform.m = alloc3DMemRefNVGPUF16(1, e->hidden, e->hidden);
+  e->wDecoder.m = nk ? alloc3DMemRefNVGPUF16(1, e->vocab, e->hidden)
+                     : alloc3DMemRefNVGPUF16(1, e->hidden, e->vocab);
+  e->t.m = alloc3DMemRefNVGPUF16(e->batch, e->seq, e->hidden);
+  e->logits.m = alloc3DMemRefNVGPUF16(e->batch, e->seq, e->vocab);
+  if (!e->wTransform.data() || !e->wDecoder.data() || !e->t.data() ||
+      !e->logits.data())
+    return -1;
+  if (e->gemmMode != 0) {
+    const int64_t M = int64_t(e->batch) * e->seq;
+    chooseGemm(e, M, e->hidden, e->hidden, e->geluForm == 1 ? 2 : 1, 0.0f,
+               &e->cTransform);
+    chooseGemm(e, M, e->vocab, e->hidden, 0, 0.0f, &e->cDecoder);
+  }
+  e->lmHead = true;
+  return 0;
+}
+
 DRV_EXPORT void homBertDestroy(HomBertEncoder *e) {
   if (!e)
     return;
@@ -235,13 +276,15 @@ DRV_EXPORT void homBertDestroy(HomBertEncoder *e) {
     w.w2.release();
   }
   for (Tensor *t : {&e->wordEmb, &e->posType, &e->ids, &e->mask, &e->cu, &e->h,
-                    &e->emb, &e->qkv, &e->attn, &e->f})
+                    &e->emb, &e->qkv, &e->attn, &e->f, &e->wTransform,
+                    &e->wDecoder, &e->t, &e->logits})
     t->release();
   delete e;
 }
 
 // which: 0 Wqkv, 1 Wo, 2 W1, 3 W2 (layer >= 0); 4 word embeddings, 5 position +
-// token-type rows (layer ignored).  `host` holds fp16 values in the layout the
+// token-type rows, 6 LM-head transform weight, 7 LM-head decoder weight (layer
+// ignored; 6 and 7 after homBertEnableLmHead).  `host` holds fp16 values in the layout the
 // tensor was allocated with ([K, N] row-major, or [N, K] when gemmMode == 0).
 DRV_EXPORT int homBertUpload(HomBertEncoder *e, int layer, int which,
                              const void *host, int64_t numel) {
@@ -251,8 +294,12 @@ DRV_EXPORT int homBertUpload(HomBertEncoder *e, int layer, int which,
       return -1;
     LayerWeights &w = e->w[size_t(layer)];
     t = which == 0 ? &w.wqkv : which == 1 ? &w.wo : which == 2 ? &w.w1 : &w.w2;
-  } else {
+  } else if (which <= 5) {
     t = which == 4 ? &e->wordEmb : &e->posType;
+  } else {
+    if (!e->lmHead || which > 7)
+      return -1;
+    t = which == 6 ? &e->wTransform : &e->wDecoder;
   }
   int64_t expect = 1;
   for (int64_t i = 0; i < t->m.rank; i++)
@@ -345,6 +392,17 @@ DRV_EXPORT int homBertGetOutput(HomBertEncoder *e, void *host) {
   const size_t n = size_t(e->batch) * e->seq * e->hidden;
   return hipOk(hipMemcpy(host, e->h.data(), n * 2, hipMemcpyDeviceToHost),
                "hipMemcpy out")
+             ? 0
+             : -1;
+}
+
+// Copy the masked-LM logits [b, s, vocab] to host.
+DRV_EXPORT int homBertGetLogits(HomBertEncoder *e, void *host) {
+  if (!e->lmHead || homBertSync(e) != 0)
+    return -1;
+  const size_t n = size_t(e->batch) * e->seq * e->vocab;
+  return hipOk(hipMemcpy(host, e->logits.data(), n * 2, hipMemcpyDeviceToHost),
+               "hipMemcpy logits")
              ? 0
              : -1;
 }

@@ -2,6 +2,7 @@
 
 #include <cstring>
 #include <mutex>
+#include <vector>
 
 namespace hom {
 
@@ -16,6 +17,8 @@ struct ScratchBuf {
   size_t bytes = 0;
 };
 ScratchBuf g_scratch[kNumSlots];
+std::vector<void *> g_retired; // replaced scratch buffers, kept allocated
+int g_scratchGeneration = 0;
 } // namespace
 
 int errorMode() { return g_errorMode; }
@@ -29,8 +32,10 @@ void recordError(const char *file, int line, const char *fmt, ...) {
   va_end(ap);
   const char *base = strrchr(file, '/');
   base = base ? base + 1 : file;
-  fprintf(stderr, "hom_amdgpu error: %s (%s:%d)\n", buf, base, line);
-  fflush(stderr);
+  if (g_errorMode != 2) {
+    fprintf(stderr, "hom_amdgpu error: %s (%s:%d)\n", buf, base, line);
+    fflush(stderr);
+  }
   if (g_errorMode == 0)
     abort();
   g_lastError = buf;
@@ -65,23 +70,25 @@ const DeviceInfo &deviceInfo() {
   return info;
 }
 
-void *scratch(ScratchSlot slot, size_t bytes, bool zero) {
+int libraryScratchGeneration() { return g_scratchGeneration; }
+
+void *libraryScratch(ScratchSlot slot, size_t bytes, bool zero) {
   ScratchBuf &b = g_scratch[slot];
   if (bytes <= b.bytes)
     return b.ptr;
-  // Growing replaces the buffer: wait for queued work that may still use the
-  // old one.  Sizes are rounded up generously so this is rare.
+  // Growing never frees the old buffer: queued kernels and captured graphs
+  // still hold its address.  It stays allocated (retired) until the process
+  // ends; sizes double, so all retired buffers together are smaller than the
+  // live one.
   size_t want = 1;
   while (want < bytes)
     want <<= 1;
-  if (b.ptr) {
-    HOM_HIP_RET(hipDeviceSynchronize(), nullptr);
-    HOM_HIP_RET(hipFree(b.ptr), nullptr);
-    b.ptr = nullptr;
-    b.bytes = 0;
-  }
   void *p = nullptr;
   HOM_HIP_RET(hipMalloc(&p, want), nullptr);
+  if (b.ptr) {
+    g_retired.push_back(b.ptr);
+    g_scratchGeneration++;
+  }
   if (zero) {
     HOM_HIP_RET(hipMemset(p, 0, want), nullptr);
   }

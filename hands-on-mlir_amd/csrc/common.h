@@ -17,7 +17,8 @@ namespace hom {
 
 // ---------------------------------------------------------------- errors --
 // mode 0: print + abort (reference behaviour); mode 1: print, remember, and
-// let the entry point return early.
+// let the entry point return early; mode 2 (library-internal, used while the
+// autotuner probes whether a kernel accepts a problem): remember silently.
 int errorMode();
 void setErrorMode(int mode);
 void recordError(const char *file, int line, const char *fmt, ...)
@@ -94,11 +95,17 @@ struct DeviceInfo {
 const DeviceInfo &deviceInfo();
 
 // Grow-only device scratch, one buffer per slot.  Slot kWorkspace holds
-// split-K partial tiles, kCounters the per-tile arrival counters (kept zero
-// between launches by the kernels themselves), kTemp short-lived temporaries.
+// split-K partial tiles, kTemp the temporaries of the layer-norm GEMM pair.
+// A buffer that has been handed out is never freed while the process lives:
+// kernels already enqueued, and HIP graphs captured earlier, keep its address
+// in their arguments.  When a slot must grow, a new buffer of at least twice
+// the size is allocated and the old one is retired (kept, unused by later
+// calls), so retired buffers add up to less than the live one.
 enum ScratchSlot { kWorkspace = 0, kCounters = 1, kTemp = 2, kNumSlots = 3 };
 // Returns nullptr (after recording an error) on allocation failure.  `zero`
 // clears newly allocated memory once, at allocation time.
-void *scratch(ScratchSlot slot, size_t bytes, bool zero);
+void *libraryScratch(ScratchSlot slot, size_t bytes, bool zero);
+// Number of times any slot has been replaced by a larger buffer (tests).
+int libraryScratchGeneration();
 
 } // namespace hom

@@ -226,7 +226,9 @@ __global__ __launch_bounds__(256) void rowStatsKernel(
   if (lane == 0) {
     const float m = s / float(n);
     const float ms = sq / float(n);
-    const float rstd = 1.0f / sqrtf(ms - m * m + eps);
+    // E[x^2] - E[x]^2 cancels to a small negative number for near-constant
+    // rows; clamped so that a tiny eps cannot turn it into a NaN
+    const float rstd = 1.0f / sqrtf(fmaxf(ms - m * m, 0.f) + eps);
     var[row] = _Float16(rstd);
     mean[row] = _Float16(-m * rstd);
   }

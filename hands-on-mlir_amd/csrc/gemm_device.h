@@ -1,0 +1,506 @@
+// Device-side building blocks shared by the fp16 GEMM kernel families
+// (gemm_dma.h, gemm_pipe.h, gemm_staged.h) and their launch plumbing.
+//
+//   D = epilogue(alpha * A.B + beta * C)
+//   A [M, K] row-major; B [K, N] row-major (or [N, K] when pre-transposed);
+//   C, D [M, N] row-major, D may alias C.
+//
+// These kernels replace the CUTLASS GemmUniversal instances the reference
+// generates (python/gemm_generator.py:237-278, python/hom_manifest.py:503-533)
+// and the cuBLASLt call behind nvteGemmF16
+// (include/NVGPUKernels/GemmRunner.h:404-425).
+//
+// Common structure
+//  * one workgroup of WM x WN wavefronts computes a BM x BN tile of D; every
+//    wavefront owns a (BM/WM) x (BN/WN) sub-tile made of 32x32 MFMA blocks
+//    (v_mfma_f32_32x32x16_f16: 64 lanes x 8 halves per operand, 16 fp32
+//    accumulators per lane);
+//  * the MFMA is issued with the operands swapped (B fragment first), i.e. it
+//    produces the transposed block, so each lane ends up with 4 consecutive
+//    columns of one row of D and the epilogue can use 64-bit accesses;
+//  * split-K: gridDim.y slices of K each store their fp32 partial tile to a
+//    workspace; a second, small kernel sums the slices in slice order
+//    (deterministic, fp32) and runs the epilogue.  Nothing spins or fences;
+//  * workgroup ids are remapped so that each of the 8 XCDs (which receive
+//    consecutive ids round-robin and have private L2s) works on a contiguous
+//    run of tiles.
+//
+// The kernel templates live in headers and are instantiated explicitly in the
+// gemm_inst_*.hip translation units (one per family / size class, so that they
+// compile in parallel); gemm.hip holds the manifest table that refers to the
+// launch functions.
+#pragma once
+
+#include "cross_lane.h"
+#include "kernels.h"
+
+#include <algorithm>
+#include <type_traits>
+#include <utility>
+
+namespace hom {
+namespace gemmk {
+
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>), unrolled.
+template <class F, int... I>
+__device__ __forceinline__ void staticForImpl(F &&f,
+                                              std::integer_sequence<int, I...>) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, class F> __device__ __forceinline__ void staticFor(F &&f) {
+  staticForImpl(f, std::make_integer_sequence<int, N>{});
+}
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+typedef float float16v __attribute__((ext_vector_type(16)));
+typedef float float4v __attribute__((ext_vector_type(4)));
+typedef float float2v __attribute__((ext_vector_type(2)));
+typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
+typedef short short4v __attribute__((ext_vector_type(4)));
+
+constexpr int kWave = 64;
+constexpr int kNumXcd = 8;
+
+#define HOM_LDS_PTR(p) ((__attribute__((address_space(3))) void *)(p))
+
+struct GemmParams {
+  const _Float16 *A;
+  const _Float16 *B;
+  const _Float16 *C;
+  _Float16 *D;
+  float *workspace; // split-K partial tiles (null when gridDim.y == 1)
+  int M, N, K;
+  int64_t lda, ldb, ldc, ldd;
+  int cRowPeriod;
+  float alpha, beta;
+  int tilesM, tilesN;
+  int kTilesPerSlice;
+  // layer-norm pair (kEpiRowStats / kEpiRowAffine kernels only)
+  float *rowStatPartials;
+  const _Float16 *rowScale;
+  const _Float16 *rowShift;
+  const float *colSum;
+  int colSumSlices;
+};
+
+// Epilogue codes beyond the three activations of the manifest kernels: linear
+// output plus row-statistic partial sums, and linear output of a per-row
+// affine transform of A folded into the accumulator.
+constexpr int kEpiRowStats = 3;
+constexpr int kEpiRowAffine = 4;
+
+// GELU(x) = 0.5 x (1 + erf(x / sqrt 2)) = max(x, 0) - 0.5 |x| erfc(|x| / sqrt 2)
+// (x >= 0: 1 + erf = 2 - erfc; x < 0: 1 + erf = erfc(|z|); no cancellation on
+// the negative side), with erfc(a / sqrt 2) = 2^P(a): P is the degree-6 least
+// squares fit of log2 erfc(a / sqrt 2) on [0, 8], weighted by the sensitivity
+// of GELU to it.  Absolute error <= 2.7e-7 over fp32 inputs (the fp32 rounding
+// of the result itself near |x| = 4), at most one fp16 ulp away from the
+// exactly rounded value.  Beyond a = 8 the factor stays at 2^P(8) ~ 1e-15.
+// Six FMAs and one exp2: the epilogue runs when no MFMA work is left to hide
+// it, so its instruction count is wall time; the library erff costs 3x this.
+__device__ __forceinline__ float geluErf(float x) {
+  const float ax = fabsf(x);
+  const float a = fminf(ax, 8.0f);
+  float P = fmaf(3.448796997e-05f, a, -7.812886615e-04f);
+  P = fmaf(P, a, 8.119936101e-03f);
+  P = fmaf(P, a, -5.347220227e-02f);
+  P = fmaf(P, a, -4.587264359e-01f);
+  P = fmaf(P, a, -1.151216269e+00f);
+  P = fmaf(P, a, 8.451195754e-06f);
+  return fmaf(-0.5f * ax, __builtin_amdgcn_exp2f(P), fmaxf(x, 0.0f));
+}
+// 0.5 x (1 + tanh(u)) == x / (1 + exp(-2u)), u = sqrt(2/pi) (x + 0.044715 x^3)
+__device__ __forceinline__ float geluTanh(float x) {
+  const float u = 0.7978845608028654f * (x + 0.044715f * x * x * x);
+  // exp(-2u) = exp2(-2 log2(e) u); large negative x gives x * rcp(inf) = -0
+  const float e = __builtin_amdgcn_exp2f(u * -2.88539008177792681472f);
+  return x * __builtin_amdgcn_rcpf(1.0f + e);
+}
+
+template <int EPI> __device__ __forceinline__ float activate(float v) {
+  if (EPI == int(Epilogue::kGeluErf))
+    return geluErf(v);
+  if (EPI == int(Epilogue::kGeluTanh))
+    return geluTanh(v);
+  return v;
+}
+
+// XCD-contiguous tile id for this workgroup.
+__device__ __forceinline__ int tileForBlock(int nTiles, int pid) {
+  const int q = nTiles / kNumXcd, r = nTiles % kNumXcd;
+  const int xcd = pid % kNumXcd, loc = pid / kNumXcd;
+  return xcd * q + (xcd < r ? xcd : r) + loc;
+}
+
+// Tile id -> (tile row, tile column).  Ids walk groups of kGroupM tile rows
+// column by column, so that the workgroups running at the same time on one XCD
+// cover a compact block of D and share both A rows and B columns in that XCD's
+// L2 instead of streaming all of B for every tile row.
+constexpr int kGroupM = 8;
+__device__ __forceinline__ void tileCoords(int tile, int tilesM, int tilesN,
+                                           int *tileM, int *tileN) {
+  const int groupSize = kGroupM * tilesN;
+  const int g = tile / groupSize;
+  const int firstM = g * kGroupM;
+  const int rows = tilesM - firstM < kGroupM ? tilesM - firstM : kGroupM;
+  const int inGroup = tile - g * groupSize;
+  *tileM = firstM + inGroup % rows;
+  *tileN = inGroup / rows;
+}
+
+// Accumulator layout shared by every kernel here (transposed 32x32 block):
+// accumulator e of lane l is column 8*(e/4) + 4*(l/32) + e%4, row l%32.
+template <int MI, int NI, int WTM, int WTN, int EPI, int VEC>
+__device__ __forceinline__ void epilogueStore(const GemmParams &p,
+                                              float16v (&acc)[MI][NI], int m0,
+                                              int n0, int waveM, int waveN,
+                                              int lane) {
+  const int l32 = lane % 32, kb = lane / 32;
+  const bool useC = p.beta != 0.f;
+  // 8-byte accesses need rows of C and D that start 8-byte aligned
+  const bool quadRows = p.ldd % 4 == 0 && (!useC || p.ldc % 4 == 0);
+#pragma unroll
+  for (int i = 0; i < MI; i++) {
+    const int m = m0 + waveM * WTM + i * 32 + l32;
+    if (m >= p.M)
+      continue;
+    const int64_t cRow = int64_t(m % p.cRowPeriod) * p.ldc;
+    const int64_t dRow = int64_t(m) * p.ldd;
+#pragma unroll
+    for (int j = 0; j < NI; j++) {
+#pragma unroll
+      for (int g = 0; g < 4; g++) {
+        const int n = n0 + waveN * WTN + j * 32 + g * 8 + kb * 4;
+        if (VEC == 8 && quadRows && n + 4 <= p.N) {
+          float c[4] = {0.f, 0.f, 0.f, 0.f};
+          if (useC) {
+            const half4 cv = *reinterpret_cast<const half4 *>(p.C + cRow + n);
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+              c[e] = float(cv[e]);
+          }
+          half4 o;
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            float v = p.alpha * acc[i][j][g * 4 + e];
+            if (useC)
+              v += p.beta * c[e];
+            o[e] = _Float16(activate<EPI>(v));
+          }
+          *reinterpret_cast<half4 *>(p.D + dRow + n) = o;
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            if (n + e < p.N) {
+              float v = p.alpha * acc[i][j][g * 4 + e];
+              if (useC)
+                v += p.beta * float(p.C[cRow + n + e]);
+              p.D[dRow + n + e] = _Float16(activate<EPI>(v));
+            }
+          }
+        }
+      }
+    }
+  }
+}
+
+// Same result as epilogueStore for 8-aligned problems, with full-width memory
+// accesses: each wavefront turns its accumulators around through a private LDS
+// strip (32 rows x WTN fp32, rows padded by 16 bytes), so that a lane ends up
+// with 8 consecutive columns of one row and reads C / writes D 16 bytes at a
+// time, a row segment of WTN halves per WTN/8 lanes.  In accumulator order a
+// store instruction scatters 16-byte pieces over 32 rows, which costs more
+// than a microsecond on a 1024 x 3072 output.  `smem` is the main loop's LDS;
+// the barrier makes sure no wavefront still reads operands from it.
+template <int MI, int NI, int WTM, int WTN, int EPI>
+__device__ __forceinline__ void
+epilogueStoreLds(const GemmParams &p, float16v (&acc)[MI][NI], int m0, int n0,
+                 int waveM, int waveN, int lane, int wave,
+                 unsigned char *smem) {
+  constexpr int ROW_B = WTN * 4 + 16;
+  constexpr int LPR = WTN / 8;  // lanes per row on the way out
+  constexpr int RPP = 64 / LPR; // rows per pass
+  unsigned char *mine = smem + wave * (32 * ROW_B);
+  const int l32 = lane % 32, kb = lane / 32;
+  const bool useC = p.beta != 0.f;
+  const int rr = lane / LPR, cc = (lane % LPR) * 8;
+  const int n = n0 + waveN * WTN + cc;
+  // 16-byte accesses need rows of C and D that start 16-byte aligned
+  const bool vec16 = p.ldd % 8 == 0 && (!useC || p.ldc % 8 == 0);
+  // Row-affine kernels: column sums of B for this lane's 8 columns (the same
+  // columns in every pass), summed over the slices they were computed in.
+  float cs[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  if constexpr (EPI == kEpiRowAffine) {
+    if (n < p.N)
+      for (int sl = 0; sl < p.colSumSlices; sl++) {
+        const float4v *src = reinterpret_cast<const float4v *>(
+            p.colSum + int64_t(sl) * p.N + n);
+        const float4v a = src[0], b = src[1];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          cs[e] += a[e];
+          cs[e + 4] += b[e];
+        }
+      }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < MI; i++) {
+#pragma unroll
+    for (int j = 0; j < NI; j++)
+#pragma unroll
+      for (int g = 0; g < 4; g++) {
+        float4v v;
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+          v[e] = acc[i][j][g * 4 + e];
+        *reinterpret_cast<float4v *>(mine + l32 * ROW_B +
+                                     (j * 32 + g * 8 + kb * 4) * 4) = v;
+      }
+#pragma unroll
+    for (int pass = 0; pass < 32 / RPP; pass++) {
+      const int r = pass * RPP + rr;
+      const float4v lo =
+          *reinterpret_cast<const float4v *>(mine + r * ROW_B + cc * 4);
+      const float4v hi =
+          *reinterpret_cast<const float4v *>(mine + r * ROW_B + cc * 4 + 16);
+      const int m = m0 + waveM * WTM + i * 32 + r;
+      float rowSum = 0.f, rowSq = 0.f;
+      if (m < p.M && n < p.N) {
+        const _Float16 *cPtr = p.C + int64_t(m % p.cRowPeriod) * p.ldc + n;
+        _Float16 *dPtr = p.D + int64_t(m) * p.ldd + n;
+        float c[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        if (useC) {
+          if (vec16) {
+            const half8 cv = *reinterpret_cast<const half8 *>(cPtr);
+#pragma unroll
+            for (int e = 0; e < 8; e++)
+              c[e] = float(cv[e]);
+          } else {
+            // rows start at 4-byte boundaries only (N not a multiple of 8):
+            // pairs, and the pair that reaches past column N is dropped (N even)
+#pragma unroll
+            for (int e = 0; e < 8; e += 2)
+              if (n + e < p.N) {
+                const half2v cv = *reinterpret_cast<const half2v *>(cPtr + e);
+                c[e] = float(cv[0]);
+                c[e + 1] = float(cv[1]);
+              }
+          }
+        }
+        float rowScale = 1.f, rowShift = 0.f;
+        if constexpr (EPI == kEpiRowAffine) {
+          rowScale = float(p.rowScale[m]);
+          rowShift = float(p.rowShift[m]);
+        }
+        half8 o;
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+          float a = e < 4 ? lo[e] : hi[e - 4];
+          if constexpr (EPI == kEpiRowAffine)
+            a = fmaf(rowScale, a, rowShift * cs[e]);
+          float v = p.alpha * a;
+          if (useC)
+            v += p.beta * c[e];
+          o[e] = _Float16(activate<EPI>(v));
+        }
+        if constexpr (EPI == kEpiRowStats) {
+          // statistics of the values as stored
+#pragma unroll
+          for (int e = 0; e < 8; e++)
+            if (n + e < p.N) {
+              const float x = float(o[e]);
+              rowSum += x;
+              rowSq = fmaf(x, x, rowSq);
+            }
+        }
+        if (vec16) {
+          *reinterpret_cast<half8 *>(dPtr) = o;
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; e += 2)
+            if (n + e < p.N) {
+              half2v ov;
+              ov[0] = o[e];
+              ov[1] = o[e + 1];
+              *reinterpret_cast<half2v *>(dPtr + e) = ov;
+            }
+        }
+      }
+      if constexpr (EPI == kEpiRowStats) {
+        // the LPR lanes of a row hold its WTN columns: one partial per row and
+        // wavefront column
+        rowSum = sumAcrossLanes<LPR>(rowSum);
+        rowSq = sumAcrossLanes<LPR>(rowSq);
+        if (lane % LPR == 0 && m < p.M) {
+          const int piece = (n0 + waveN * WTN) / WTN;
+          float2v st;
+          st[0] = rowSum;
+          st[1] = rowSq;
+          *reinterpret_cast<float2v *>(p.rowStatPartials +
+                                       (int64_t(piece) * p.M + m) * 2) = st;
+        }
+      }
+    }
+  }
+}
+
+// Partial tile of one K slice -> workspace, in accumulator order (coalesced
+// 128-bit stores; the reduce kernel uses the same thread -> element mapping).
+template <int MI, int NI, int THREADS>
+__device__ __forceinline__ void storePartial(const GemmParams &p,
+                                             float16v (&acc)[MI][NI], int tile,
+                                             int slice, int numSlices,
+                                             int tid) {
+  constexpr int ACC_V4 = MI * NI * 4;
+  float4v *mine = reinterpret_cast<float4v *>(p.workspace) +
+                  (int64_t(tile) * numSlices + slice) * (ACC_V4 * THREADS);
+#pragma unroll
+  for (int i = 0; i < MI; i++)
+#pragma unroll
+    for (int j = 0; j < NI; j++)
+#pragma unroll
+      for (int g = 0; g < 4; g++) {
+        float4v v;
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+          v[e] = acc[i][j][g * 4 + e];
+        mine[((i * NI + j) * 4 + g) * THREADS + tid] = v;
+      }
+}
+
+template <int BM, int BN, int WM, int WN, int EPI, int VEC>
+__global__ __launch_bounds__(WM *WN *kWave) void splitKReduceKernel(
+    GemmParams p, int numSlices) {
+  constexpr int THREADS = WM * WN * kWave;
+  constexpr int WTM = BM / WM, WTN = BN / WN;
+  constexpr int MI = WTM / 32, NI = WTN / 32;
+  constexpr int ACC_V4 = MI * NI * 4;
+  const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+  const int tile = blockIdx.x;
+  int tileM, tileN;
+  tileCoords(tile, p.tilesM, p.tilesN, &tileM, &tileN);
+  float16v acc[MI][NI];
+#pragma unroll
+  for (int i = 0; i < MI; i++)
+#pragma unroll
+    for (int j = 0; j < NI; j++)
+#pragma unroll
+      for (int e = 0; e < 16; e++)
+        acc[i][j][e] = 0.f;
+  const float4v *ws = reinterpret_cast<const float4v *>(p.workspace) +
+                      int64_t(tile) * numSlices * (ACC_V4 * THREADS);
+  for (int s = 0; s < numSlices; s++) {
+    const float4v *part = ws + int64_t(s) * (ACC_V4 * THREADS);
+#pragma unroll
+    for (int i = 0; i < MI; i++)
+#pragma unroll
+      for (int j = 0; j < NI; j++)
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+          const float4v v = part[((i * NI + j) * 4 + g) * THREADS + tid];
+#pragma unroll
+          for (int e = 0; e < 4; e++)
+            acc[i][j][g * 4 + e] += v[e];
+        }
+  }
+  epilogueStore<MI, NI, WTM, WTN, EPI, VEC>(p, acc, tileM * BM, tileN * BN,
+                                            wave / WN, wave % WN, lane);
+}
+
+// ===================================================================== dma ==
+// Swizzles (in units of 16-byte chunks / 64-byte groups inside an LDS row).
+// K-contiguous tiles (A, and B given as [N, K]): rows of 128 bytes = 8 chunks;
+// chunk c of row r lives at position c ^ ((r >> 1) & 7), which makes the
+// 128-bit fragment reads of 16 consecutive rows hit 16 distinct bank groups.
+__device__ __forceinline__ int swzK(int row, int chunk) {
+  return chunk ^ ((row >> 1) & 7);
+}
+// Row-major B tiles: a transposing read touches rows k..k+3 and k+8..k+11, 64
+// bytes of each; 64-byte group g of row k lives at position g ^ f(k).
+template <int BN> __device__ __forceinline__ int swzN(int k, int group) {
+  if (BN == 64)
+    return group ^ ((k >> 1) & 1);
+  return group ^ (k & 3);
+}
+
+// ------------------------------------------------------------ kernel table --
+struct LaunchPlan {
+  GemmParams p;
+  int splitK;
+  int64_t nTiles;
+};
+
+template <int BM, int BN, int BK>
+Status planLaunch(const GemmProblem &pr, LaunchPlan *plan) {
+  GemmParams &p = plan->p;
+  p.A = pr.A;
+  p.B = pr.B;
+  p.C = pr.C;
+  p.D = pr.D;
+  p.M = int(pr.M);
+  p.N = int(pr.N);
+  p.K = int(pr.K);
+  p.lda = pr.lda;
+  p.ldb = pr.ldb;
+  p.ldc = pr.ldc;
+  p.ldd = pr.ldd;
+  p.cRowPeriod = int(pr.cRowPeriod > 0 ? pr.cRowPeriod : 1);
+  p.alpha = pr.alpha;
+  p.beta = pr.beta;
+  p.rowStatPartials = pr.rowStatPartials;
+  p.rowScale = pr.rowScale;
+  p.rowShift = pr.rowShift;
+  p.colSum = pr.colSum;
+  p.colSumSlices = pr.colSumSlices;
+  p.tilesM = int((pr.M + BM - 1) / BM);
+  p.tilesN = int((pr.N + BN - 1) / BN);
+  const int kTiles = int((pr.K + BK - 1) / BK);
+  int splitK = pr.splitK < 1 ? 1 : pr.splitK;
+  if (splitK > kTiles)
+    splitK = kTiles > 0 ? kTiles : 1;
+  p.kTilesPerSlice = (kTiles + splitK - 1) / splitK;
+  if (p.kTilesPerSlice > 0) // drop slices that rounding up left empty
+    splitK = (kTiles + p.kTilesPerSlice - 1) / p.kTilesPerSlice;
+  if (splitK < 1)
+    splitK = 1;
+  plan->splitK = splitK;
+  plan->nTiles = int64_t(p.tilesM) * p.tilesN;
+  HOM_CHECK_RET(plan->nTiles < (int64_t(1) << 30), Status::kInvalidArgument,
+                "gemm: too many output tiles (%lld)", (long long)plan->nTiles);
+  p.workspace = nullptr;
+  if (splitK > 1) {
+    const size_t wsBytes =
+        size_t(plan->nTiles) * splitK * size_t(BM) * BN * sizeof(float);
+    p.workspace =
+        static_cast<float *>(libraryScratch(kWorkspace, wsBytes, false));
+    if (!p.workspace)
+      return Status::kInternal;
+  }
+  return Status::kSuccess;
+}
+
+template <typename K> Status allowLds(K kernel, int bytes, bool *done) {
+  if (!*done && bytes > 48 * 1024) {
+    HOM_HIP_RET(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    bytes),
+                Status::kInternal);
+  }
+  *done = true;
+  return Status::kSuccess;
+}
+
+template <int BM, int BN, int WM, int WN, int EPI, int VEC>
+Status launchReduce(const LaunchPlan &plan, hipStream_t s) {
+  splitKReduceKernel<BM, BN, WM, WN, EPI, VEC>
+      <<<dim3((unsigned)plan.nTiles), dim3(WM * WN * kWave), 0, s>>>(
+          plan.p, plan.splitK);
+  HOM_HIP_RET(hipGetLastError(), Status::kInternal);
+  return Status::kSuccess;
+}
+
+} // namespace gemmk
+} // namespace hom

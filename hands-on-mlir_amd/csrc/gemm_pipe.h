@@ -1,0 +1,460 @@
+#pragma once
+
+#include "gemm_device.h"
+
+namespace hom {
+namespace gemmk {
+
+// ==================================================================== pipe ==
+// Same LDS layout, fragment reads and barrier placement as the dma kernels, but
+// the slabs travel global -> registers -> LDS (two LDS buffers): the loads of
+// slab i+1 are issued before slab i is multiplied and written to LDS after it.
+// The vector memory path into registers sustains several times the bandwidth
+// of the LDS-DMA path on this chip, which matters once a CU streams more than
+// ~16 bytes per clock (large tiles, or several workgroups per CU).
+template <int BM, int BN, int WM, int WN, int DIST, int EPI, bool B_NK>
+__global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(GemmParams p) {
+  static_assert(DIST >= 1, "at least one slab of global loads in flight");
+  constexpr int BK = 64;
+  constexpr int THREADS = WM * WN * kWave;
+  constexpr int WTM = BM / WM, WTN = BN / WN;
+  constexpr int MI = WTM / 32, NI = WTN / 32;
+  constexpr int A_BYTES = BM * BK * 2, B_BYTES = BN * BK * 2;
+  constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
+  constexpr int A_VECS = A_BYTES / 16, B_VECS = B_BYTES / 16;
+  static_assert(A_VECS % THREADS == 0 && B_VECS % THREADS == 0,
+                "tile must split evenly over the threads");
+  constexpr int A_PER_T = A_VECS / THREADS, B_PER_T = B_VECS / THREADS;
+  constexpr int B_ROW_BYTES = B_NK ? 128 : BN * 2;
+  constexpr int B_VPR = B_ROW_BYTES / 16; // vectors per LDS row of B
+  constexpr int KSTEPS = BK / 16;
+
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+
+  const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+  const int waveM = wave / WN, waveN = wave % WN;
+  const int l32 = lane % 32, kb = lane / 32;
+
+  // Persistent over tiles: the grid holds at most as many workgroups as fit on
+  // the chip at once and each walks tiles pid, pid + grid, ...  (the grid is a
+  // multiple of the XCD count, so a workgroup's tiles stay in its XCD's
+  // contiguous range).  A tile's output stores drain and the next tile's first
+  // slabs arrive while other work runs, instead of between two workgroups.
+  const int nTiles = p.tilesM * p.tilesN;
+  for (int vpid = blockIdx.x; vpid < nTiles; vpid += gridDim.x) {
+  if (vpid != int(blockIdx.x))
+    __syncthreads(); // the previous tile's epilogue strips live in this LDS
+  const int tile = tileForBlock(nTiles, vpid);
+  int tileM, tileN;
+  tileCoords(tile, p.tilesM, p.tilesN, &tileM, &tileN);
+  const int m0 = tileM * BM, n0 = tileN * BN;
+  const int slice = blockIdx.y, numSlices = gridDim.y;
+  const int kTiles = (p.K + BK - 1) / BK;
+  const int ktBegin = slice * p.kTilesPerSlice;
+  int ktEnd = ktBegin + p.kTilesPerSlice;
+  if (ktEnd > kTiles)
+    ktEnd = kTiles;
+
+  // ---- global sources ----
+  // Buffer loads from descriptors based at this tile's first row (A) / first
+  // row or column block (B): a constant 32-bit byte offset per thread plus a
+  // scalar offset per slab.  Rows / columns past the edge are clamped to the
+  // last valid one: what they fetch only reaches outputs that are never
+  // stored.  Every slab issues the same number of loads and there is no branch
+  // around a load, so the compiler's outstanding-load counts are exact (a
+  // branch makes it wait for everything in flight and defeats the pipeline).
+  // The main loop walks the slice's FULL slabs only and asks for no range
+  // test per vector: vector instructions in that loop cost matrix-core time.
+  // A slab requested past the last full one is replaced by the last full one
+  // (it is never used), and a partial last slab (K not a multiple of 64) is
+  // multiplied ahead of the loop by a short unpipelined pass whose loads map
+  // vectors at or past kEnd to an offset outside the descriptor (they read as
+  // zero without touching memory).
+  constexpr uint32_t kOob = 0x80000000u;
+  auto clampBytes = [](int64_t b) -> int32_t {
+    return b > 0x7fffffffLL ? 0x7fffffff : (b < 0 ? 0 : int32_t(b));
+  };
+  const _Float16 *aTile = p.A + int64_t(m0) * p.lda;
+  const auto rsrcA = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<_Float16 *>(aTile), 0,
+      clampBytes(int64_t(p.M - m0) * p.lda * 2), 0x00020000);
+  const _Float16 *bTile = B_NK ? p.B + int64_t(n0) * p.ldb : p.B + n0;
+  const auto rsrcB = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<_Float16 *>(bTile), 0,
+      clampBytes(B_NK ? int64_t(p.N - n0) * p.ldb * 2
+                      : (int64_t(p.K) * p.ldb - n0) * 2),
+      0x00020000);
+  const int kEnd = ktEnd * BK < p.K ? ktEnd * BK : p.K;
+  uint32_t aOff[A_PER_T], bOff[B_PER_T];
+  // LDS destination of vector i = destination of vector 0 + i * DST_STEP: the
+  // row advances by a multiple of 16 per vector, which leaves both swizzles
+  // unchanged (they depend on row bits 0..3 only).
+  constexpr int DST_STEP = THREADS * 16;
+  static_assert((THREADS / 8) % 16 == 0 && (THREADS / B_VPR) % 4 == 0 &&
+                    (BN != 64 || (THREADS / B_VPR) % 4 == 0),
+                "vector step must preserve the LDS swizzles");
+  int aDst0 = 0, bDst0 = 0;
+  int aK[A_PER_T], bK[B_PER_T]; // k position inside the slab
+#pragma unroll
+  for (int i = 0; i < A_PER_T; i++) {
+    const int v = tid + i * THREADS;
+    const int r = v / 8, c = v % 8;
+    const int rr = m0 + r < p.M ? r : p.M - 1 - m0;
+    aK[i] = c * 8;
+    aOff[i] = (uint32_t(rr) * uint32_t(p.lda) + c * 8) * 2u;
+    if (i == 0)
+      aDst0 = r * 128 + swzK(r, c) * 16;
+  }
+#pragma unroll
+  for (int i = 0; i < B_PER_T; i++) {
+    const int v = tid + i * THREADS;
+    const int r = v / B_VPR, c = v % B_VPR;
+    if (B_NK) {
+      const int rr = n0 + r < p.N ? r : p.N - 1 - n0;
+      bK[i] = c * 8;
+      bOff[i] = (uint32_t(rr) * uint32_t(p.ldb) + c * 8) * 2u;
+      if (i == 0)
+        bDst0 = r * 128 + swzK(r, c) * 16;
+    } else {
+      const int cc = n0 + c * 8 < p.N ? c * 8 : p.N - 8 - n0;
+      bK[i] = r;
+      bOff[i] = (uint32_t(r) * uint32_t(p.ldb) + cc) * 2u;
+      if (i == 0)
+        bDst0 = r * B_ROW_BYTES + swzN<BN>(r, c / 4) * 64 + (c % 4) * 16;
+    }
+  }
+
+  half8 regA[DIST][A_PER_T], regB[DIST][B_PER_T];
+  // Slabs of this slice that lie inside [0, kEnd) entirely, and whether a
+  // partial one follows them (only the last slice of a ragged K has one).
+  const int nkFull = (kEnd - ktBegin * BK) / BK;
+  const bool hasTail = kEnd - ktBegin * BK > nkFull * BK;
+  const int ktLastFull = ktBegin + nkFull - 1;
+  // Full slab kt (requests past the last full slab fetch that one again).
+  auto loadGlobal = [&](int kt, auto setC) {
+    constexpr int S = decltype(setC)::value;
+    const int k0 = (kt < ktLastFull ? kt : ktLastFull) * BK;
+    const uint32_t sA = uint32_t(k0) * 2u;
+    const uint32_t sB = B_NK ? sA : uint32_t(k0) * uint32_t(p.ldb) * 2u;
+#pragma unroll
+    for (int i = 0; i < A_PER_T; i++)
+      regA[S][i] = __builtin_bit_cast(
+          half8, __builtin_amdgcn_raw_buffer_load_b128(rsrcA, aOff[i], sA, 0));
+#pragma unroll
+    for (int i = 0; i < B_PER_T; i++)
+      regB[S][i] = __builtin_bit_cast(
+          half8, __builtin_amdgcn_raw_buffer_load_b128(rsrcB, bOff[i], sB, 0));
+  };
+  // Slab kt with a range test per vector (the partial slab).
+  auto loadGlobalChecked = [&](int kt, auto setC) {
+    constexpr int S = decltype(setC)::value;
+    const int k0 = kt * BK;
+    const uint32_t sA = uint32_t(k0) * 2u;
+    const uint32_t sB = B_NK ? sA : uint32_t(k0) * uint32_t(p.ldb) * 2u;
+#pragma unroll
+    for (int i = 0; i < A_PER_T; i++)
+      regA[S][i] = __builtin_bit_cast(
+          half8, __builtin_amdgcn_raw_buffer_load_b128(
+                     rsrcA, k0 + aK[i] < kEnd ? aOff[i] : kOob, sA, 0));
+#pragma unroll
+    for (int i = 0; i < B_PER_T; i++)
+      regB[S][i] = __builtin_bit_cast(
+          half8, __builtin_amdgcn_raw_buffer_load_b128(
+                     rsrcB, k0 + bK[i] < kEnd ? bOff[i] : kOob, sB, 0));
+  };
+  auto storeLds = [&](int stage, auto setC) {
+    constexpr int S = decltype(setC)::value;
+    unsigned char *sA = smem + stage * STAGE_BYTES;
+    unsigned char *sB = sA + A_BYTES;
+#pragma unroll
+    for (int i = 0; i < A_PER_T; i++)
+      *reinterpret_cast<half8 *>(sA + aDst0 + i * DST_STEP) = regA[S][i];
+#pragma unroll
+    for (int i = 0; i < B_PER_T; i++)
+      *reinterpret_cast<half8 *>(sB + bDst0 + i * DST_STEP) = regB[S][i];
+  };
+
+  float16v acc[MI][NI];
+#pragma unroll
+  for (int i = 0; i < MI; i++)
+#pragma unroll
+    for (int j = 0; j < NI; j++)
+#pragma unroll
+      for (int e = 0; e < 16; e++)
+        acc[i][j][e] = 0.f;
+
+  // ---- fragment addresses: a few per-lane bases, the rest are immediates ----
+  // K-contiguous tiles: the swizzle term (row >> 1) & 7 only involves bits of
+  // lane % 32 (wave / block offsets are multiples of 32), so the chunk position
+  // of k step kk is the same for every 32-row block of the wavefront.
+  const int swzLane = (l32 >> 1) & 7;
+  int aFrag[KSTEPS], bFragK[KSTEPS];
+#pragma unroll
+  for (int kk = 0; kk < KSTEPS; kk++) {
+    aFrag[kk] = (waveM * WTM + l32) * 128 + ((kk * 2 + kb) ^ swzLane) * 16;
+    bFragK[kk] =
+        A_BYTES + (waveN * WTN + l32) * 128 + ((kk * 2 + kb) ^ swzLane) * 16;
+  }
+  // Row-major B, transposing reads: source lane L = lane % 16 of a 16-lane group
+  // supplies row kbase + L/4 and the 4 columns at (L%4)*4 of the group's 16
+  // columns.  k & 3 == L/4 for every (kk, kb, h), so the 64-byte group swizzle
+  // is a per-lane constant as well.
+  const int trRow = (lane % 16) / 4;
+  const int trCol = ((lane % 32) / 16) * 16 + (lane % 4) * 4;
+  int bFragN[NI];
+#pragma unroll
+  for (int j = 0; j < NI; j++) {
+    const int group = (waveN * WTN) / 32 + j;
+    bFragN[j] = A_BYTES + (kb * 8 + trRow) * B_ROW_BYTES +
+                swzN<BN>(trRow, group) * 64 + trCol * 2;
+  }
+
+  // One fragment per call: unit u < MI is A block u, the rest are B blocks.
+  auto loadFragUnit = [&](int stage, int kk, half8 (&fa)[MI], half8 (&fb)[NI],
+                          auto uC) {
+    constexpr int U = decltype(uC)::value;
+    const unsigned char *st = smem + stage * STAGE_BYTES;
+    if constexpr (U < MI) {
+      fa[U] = *reinterpret_cast<const half8 *>(st + aFrag[kk] + U * 32 * 128);
+    } else if constexpr (B_NK) {
+      constexpr int j = U - MI;
+      fb[j] = *reinterpret_cast<const half8 *>(st + bFragK[kk] + j * 32 * 128);
+    } else {
+      constexpr int j = U - MI;
+      short4v t[2];
+#pragma unroll
+      for (int h = 0; h < 2; h++)
+        t[h] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (__attribute__((address_space(3))) short4v *)(
+                st + bFragN[j] + (kk * 16 + h * 4) * B_ROW_BYTES));
+      typedef short short8v __attribute__((ext_vector_type(8)));
+      short8v both;
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        both[e] = t[0][e];
+        both[4 + e] = t[1][e];
+      }
+      fb[j] = __builtin_bit_cast(half8, both);
+    }
+  };
+  auto loadFrags = [&](int stage, int kk, half8 (&fa)[MI], half8 (&fb)[NI]) {
+    staticFor<MI + NI>([&](auto uC) { loadFragUnit(stage, kk, fa, fb, uC); });
+  };
+
+  // ---- main loop ----
+  // LDS holds slab i (buffer i & 1); slabs i+1 .. i+DIST sit in registers or are
+  // on their way there, slab s in register set s % DIST.  While slab i is
+  // multiplied, slab i+1 moves from its register set to the other LDS buffer
+  // one 16-byte vector at a time, and each vector's registers are refilled
+  // with slab i+1+DIST right behind the LDS write.  These LDS writes and global
+  // loads are spread between the MFMAs of the first KSTEPS-1 k steps
+  // (scheduling barriers pin the order): issued as one burst they fill the
+  // memory pipelines' queues, the wavefront blocks on issue, and with both
+  // wavefronts of a SIMD in the same phase the matrix core idles for as long as
+  // the burst takes to drain.  The loop is unrolled DIST times to keep the
+  // register-set index a compile-time constant.
+  // The barrier is a bare s_barrier behind an LDS-only wait: a fence here would
+  // drain the global loads that were just issued.
+  // The fragments of k step kk+1 are fetched under the MFMAs of step kk (two
+  // fragment sets).
+  constexpr int NV = A_PER_T + B_PER_T; // vectors per thread and slab
+  constexpr int NM = MI * NI;           // MFMAs per wavefront and k step
+  constexpr int ST_STEPS = KSTEPS - 1;  // k steps that carry staging work
+  half8 fa[2][MI], fb[2][NI];
+  const int nk = nkFull; // the pipelined loop walks the full slabs
+  // Moves vector v of register set S to LDS and refills it from full slab kt
+  // (already clamped to the last full slab by the caller).
+  auto stageVec = [&](int stage, int kt, auto setC, auto vC) {
+    constexpr int S = decltype(setC)::value;
+    constexpr int V = decltype(vC)::value;
+    unsigned char *sA = smem + stage * STAGE_BYTES;
+    unsigned char *sB = sA + A_BYTES;
+    const int k0 = kt * BK;
+    if constexpr (V < A_PER_T) {
+      *reinterpret_cast<half8 *>(sA + aDst0 + V * DST_STEP) = regA[S][V];
+      regA[S][V] = __builtin_bit_cast(
+          half8, __builtin_amdgcn_raw_buffer_load_b128(rsrcA, aOff[V],
+                                                       uint32_t(k0) * 2u, 0));
+    } else {
+      constexpr int W = V - A_PER_T;
+      *reinterpret_cast<half8 *>(sB + bDst0 + W * DST_STEP) = regB[S][W];
+      regB[S][W] = __builtin_bit_cast(
+          half8,
+          __builtin_amdgcn_raw_buffer_load_b128(
+              rsrcB, bOff[W],
+              B_NK ? uint32_t(k0) * 2u : uint32_t(k0) * uint32_t(p.ldb) * 2u,
+              0));
+    }
+  };
+  // The MFMAs of one k step on fragments (a, b).  Spread between them: the
+  // fragment reads of another k step (rdStage, rdKk) into (na, nb) when RD, and
+  // the staging vectors [V0, V1) when stageOn.  Memory operation q of n goes in
+  // front of MFMA q * NM / n.
+  auto mfmaMixed = [&](half8 (&a)[MI], half8 (&b)[NI], half8 (&na)[MI],
+                       half8 (&nb)[NI], int rdStage, int rdKk, auto rdC,
+                       int stStage, int kt, bool stageOn, auto setC, auto v0C,
+                       auto v1C) {
+    constexpr bool RD = decltype(rdC)::value;
+    constexpr int V0 = decltype(v0C)::value, V1 = decltype(v1C)::value;
+    constexpr int NR = RD ? MI + NI : 0;
+    constexpr int N = NR + (V1 - V0);
+    staticFor<NM>([&](auto mC) {
+      constexpr int m = decltype(mC)::value;
+      if constexpr (N > 0) {
+        staticFor<N>([&](auto qC) {
+          constexpr int q = decltype(qC)::value;
+          if constexpr (q * NM / N == m) {
+            __builtin_amdgcn_sched_barrier(0);
+            if constexpr (q < NR) {
+              loadFragUnit(rdStage, rdKk, na, nb,
+                           std::integral_constant<int, (q < NR ? q : 0)>{});
+            } else {
+              if (stageOn)
+                stageVec(stStage, kt, setC,
+                         std::integral_constant<int, V0 + q - NR>{});
+            }
+            __builtin_amdgcn_sched_barrier(0);
+          }
+        });
+      }
+      acc[m / NI][m % NI] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+          b[m % NI], a[m / NI], acc[m / NI][m % NI], 0, 0, 0);
+    });
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  // tailC: the slab may be the last one (then nothing follows it); the
+  // steady-state loop knows it is not and runs without branches.
+  auto slab = [&](int i, auto setC, auto tailC) {
+    constexpr bool kTail = decltype(tailC)::value;
+    const int cur = i & 1;
+    const bool more = !kTail || i + 1 < nk;
+    const int ktWant = ktBegin + i + 1 + DIST;
+    const int ktNext = ktWant < ktLastFull ? ktWant : ktLastFull;
+    staticFor<KSTEPS>([&](auto kkC) {
+      constexpr int kk = decltype(kkC)::value;
+      constexpr int V0 = kk < ST_STEPS ? kk * NV / ST_STEPS : NV;
+      constexpr int V1 = kk < ST_STEPS ? (kk + 1) * NV / ST_STEPS : NV;
+      using V0C = std::integral_constant<int, V0>;
+      using V1C = std::integral_constant<int, V1>;
+      constexpr int cs = kk % 2, ns = (kk + 1) % 2;
+      if constexpr (kk < KSTEPS - 1) {
+        mfmaMixed(fa[cs], fb[cs], fa[ns], fb[ns], cur, kk + 1, std::true_type{},
+                  cur ^ 1, ktNext, more, setC, V0C{}, V1C{});
+      } else {
+        static_assert(ns == 0, "the next slab finds its first fragments in set 0");
+        if (more) {
+          // Every wavefront has its last fragments of slab i in registers and
+          // slab i+1 is complete in the other buffer after this barrier; its
+          // first fragments arrive under the MFMAs of the last k step.
+          asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+          mfmaMixed(fa[cs], fb[cs], fa[ns], fb[ns], cur ^ 1, 0, std::true_type{},
+                    0, 0, false, setC, V0C{}, V1C{});
+        } else {
+          mfmaMixed(fa[cs], fb[cs], fa[ns], fb[ns], 0, 0, std::false_type{}, 0,
+                    0, false, setC, V0C{}, V1C{});
+        }
+      }
+    });
+  };
+  if (hasTail) {
+    // The partial slab, unpipelined: it is one slab of a ragged problem.
+    using Set0 = std::integral_constant<int, 0>;
+    loadGlobalChecked(ktBegin + nkFull, Set0{});
+    storeLds(0, Set0{});
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < KSTEPS; kk++) {
+      loadFrags(0, kk, fa[0], fb[0]);
+#pragma unroll
+      for (int m = 0; m < NM; m++)
+        acc[m / NI][m % NI] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+            fb[0][m % NI], fa[0][m / NI], acc[m / NI][m % NI], 0, 0, 0);
+    }
+    __syncthreads(); // buffer 0 is rewritten by the first full slab
+  }
+  if (nk > 0) {
+    staticFor<DIST>(
+        [&](auto d) { loadGlobal(ktBegin + decltype(d)::value, d); });
+    storeLds(0, std::integral_constant<int, 0>{});
+    loadGlobal(ktBegin + DIST, std::integral_constant<int, 0>{});
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    loadFrags(0, 0, fa[0], fb[0]);
+    int i = 0;
+    for (; i + DIST < nk; i += DIST) {
+      staticFor<DIST>([&](auto d) {
+        constexpr int D = decltype(d)::value;
+        slab(i + D, std::integral_constant<int, (D + 1) % DIST>{},
+             std::false_type{});
+      });
+    }
+    bool go = true;
+    staticFor<DIST>([&](auto d) {
+      constexpr int D = decltype(d)::value;
+      go = go && i + D < nk;
+      if (go)
+        slab(i + D, std::integral_constant<int, (D + 1) % DIST>{},
+             std::true_type{});
+    });
+  }
+
+  if (numSlices > 1) {
+    storePartial<MI, NI, THREADS>(p, acc, tile, slice, numSlices, tid);
+    continue;
+  }
+  static_assert(WM * WN * 32 * (WTN * 4 + 16) <= 2 * STAGE_BYTES,
+                "epilogue strips must fit the main loop's LDS");
+  epilogueStoreLds<MI, NI, WTM, WTN, EPI>(p, acc, m0, n0, waveM, waveN, lane,
+                                          wave, smem);
+  } // tiles of this workgroup
+}
+
+template <int BM, int BN, int WM, int WN, int DIST, int EPI, bool B_NK>
+Status launchPipe(const GemmProblem &pr, hipStream_t s) {
+  constexpr int SMEM = 2 * (BM + BN) * 64 * 2;
+  LaunchPlan plan;
+  Status st = planLaunch<BM, BN, 64>(pr, &plan);
+  if (st != Status::kSuccess)
+    return st;
+  // 32-bit buffer offsets: a row-major B slab is addressed from the matrix base.
+  HOM_CHECK_RET(B_NK || pr.K * pr.ldb * 2 < (int64_t(1) << 31),
+                Status::kInvalidArgument,
+                "gemm: B larger than 2 GiB is not supported by this kernel");
+  HOM_CHECK_RET((int64_t(BM) * pr.lda + pr.K) * 2 < (int64_t(1) << 31) &&
+                    (int64_t(BN) * pr.ldb + pr.K) * 2 < (int64_t(1) << 31),
+                Status::kInvalidArgument, "gemm: leading dimension too large");
+  auto kernel = gemmPipeKernel<BM, BN, WM, WN, DIST, EPI, B_NK>;
+  static bool attrSet = false;
+  st = allowLds(kernel, SMEM, &attrSet);
+  if (st != Status::kSuccess)
+    return st;
+  if (plan.nTiles == 0)
+    return Status::kSuccess;
+  // Workgroups that fit on the chip at once (rounded down to a multiple of the
+  // XCD count, which the tile order relies on); more tiles than that are walked
+  // by the same workgroups.
+  static int resident = 0;
+  if (resident == 0) {
+    int perCu = 0;
+    HOM_HIP_RET(hipOccupancyMaxActiveBlocksPerMultiprocessor(
+                    &perCu, kernel, WM * WN * kWave, SMEM),
+                Status::kInternal);
+    const int cus = deviceInfo().computeUnits > 0 ? deviceInfo().computeUnits : 256;
+    resident = perCu > 0 ? perCu * cus / kNumXcd * kNumXcd : 0;
+    if (resident < kNumXcd)
+      resident = 1 << 30; // unknown: one workgroup per tile
+  }
+  int64_t gridX = plan.nTiles;
+  if (gridX * plan.splitK > resident)
+    gridX = std::max<int64_t>(kNumXcd, resident / plan.splitK / kNumXcd * kNumXcd);
+  if (gridX > plan.nTiles)
+    gridX = plan.nTiles;
+  kernel<<<dim3((unsigned)gridX, (unsigned)plan.splitK), dim3(WM * WN * kWave),
+           SMEM, s>>>(plan.p);
+  HOM_HIP_RET(hipGetLastError(), Status::kInternal);
+  if (plan.splitK > 1)
+    return launchReduce<BM, BN, WM, WN, EPI, 8>(plan, s);
+  return Status::kSuccess;
+}
+
+} // namespace gemmk
+} // namespace hom

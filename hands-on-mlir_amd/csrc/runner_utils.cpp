@@ -176,8 +176,9 @@ void homSetStream(void *hipStream) {
   setStream(static_cast<hipStream_t>(hipStream));
 }
 void *homGetStream(void) { return static_cast<void *>(stream()); }
-void homSetErrorMode(int32_t mode) { setErrorMode(mode); }
+void homSetErrorMode(int32_t mode) { setErrorMode(mode == 1 ? 1 : 0); }
 const char *homGetLastError(void) { return takeLastError(); }
+int32_t homScratchGeneration(void) { return libraryScratchGeneration(); }
 
 void homAddLayernormF16(int64_t rankX, void *dstX, int64_t rankRes,
                         void *dstRes, int64_t rankGamma, void *dstGamma,
@@ -223,6 +224,22 @@ void homGemmProfile(int64_t M, int64_t N, int64_t K, int64_t activation,
   if (!g_profiler)
     g_profiler = new GemmProfiler(M, N, K, activation, alpha, beta);
   auto res = g_profiler->profile(M, N, K, activation, alpha, beta);
+  if (bestIdx)
+    *bestIdx = std::get<0>(res);
+  if (bestSplitK)
+    *bestSplitK = std::get<1>(res);
+  if (bestTimeMs)
+    *bestTimeMs = g_profiler->bestTimeMs();
+}
+
+void homGemmProfileLayout(int64_t M, int64_t N, int64_t K, int64_t activation,
+                          float alpha, float beta, int32_t bIsNK,
+                          int64_t *bestIdx, int32_t *bestSplitK,
+                          float *bestTimeMs) {
+  if (!g_profiler)
+    g_profiler = new GemmProfiler(M, N, K, activation, alpha, beta);
+  auto res =
+      g_profiler->profileLayout(M, N, K, activation, alpha, beta, bIsNK != 0);
   if (bestIdx)
     *bestIdx = std::get<0>(res);
   if (bestSplitK)

@@ -176,6 +176,9 @@ int fallbackKernel(Epilogue epi, int cls) {
   return findKernel(64, 64, 32, epi, 1);
 }
 
+// Kernel and split-K (stored into pr) the [N, K]-B path runs for a problem.
+int chooseNvteKernel(GemmProblem *pr, int64_t activation);
+
 } // namespace
 
 bool selectGemm(int64_t M, int64_t N, int64_t K, int64_t activation,
@@ -317,6 +320,36 @@ Status runGemmManifest(int64_t rankA, void *dstA, int64_t rankB, void *dstB,
   return launchGemm(idx, pr, stream());
 }
 
+namespace {
+int chooseNvteKernel(GemmProblem *pr, int64_t activation) {
+  int64_t sel;
+  int32_t sk;
+  const Epilogue epi = epilogueFor(activation, true);
+  selectGemm(pr->M, pr->N, pr->K, epi == Epilogue::kGeluTanh ? 2 : activation,
+             &sel, &sk);
+  int idx = int(sel);
+  pr->splitK = sk;
+  // Profiling knob: HOM_NVTE_GEMM_KERNEL="<manifest name>[,<splitK>]" pins the
+  // kernel used on this path (the epilogue must match the activation).
+  if (const char *force = getenv("HOM_NVTE_GEMM_KERNEL")) {
+    std::string f(force);
+    const size_t comma = f.find(',');
+    const std::string name = f.substr(0, comma);
+    for (int i = 0; i < gemmKernelCount(); i++)
+      if (name == gemmKernelInfo(i).name && gemmKernelInfo(i).epilogue == epi) {
+        idx = i;
+        pr->splitK = comma == std::string::npos ? 1 : atoi(f.c_str() + comma + 1);
+      }
+  }
+  const int cls = alignmentClass(*pr);
+  if (!kernelFits(gemmKernelInfo(idx), cls)) {
+    idx = fallbackKernel(epi, cls);
+    pr->splitK = 1;
+  }
+  return idx;
+}
+} // namespace
+
 Status runGemmNvte(int64_t rankA, void *dstA, bool transa, int64_t rankB,
                    void *dstB, bool transb, int64_t rankC, void *dstC,
                    int64_t rankD, void *dstD, int64_t activation, float alpha,
@@ -346,31 +379,7 @@ Status runGemmNvte(int64_t rankA, void *dstA, bool transa, int64_t rankB,
   }
   pr.alpha = alpha;
   pr.beta = beta;
-  int64_t sel;
-  int32_t sk;
-  const Epilogue epi = epilogueFor(activation, true);
-  selectGemm(pr.M, pr.N, pr.K, epi == Epilogue::kGeluTanh ? 2 : activation,
-             &sel, &sk);
-  int idx = int(sel);
-  pr.splitK = sk;
-  // Profiling knob: HOM_NVTE_GEMM_KERNEL="<manifest name>[,<splitK>]" pins the
-  // kernel used on this path (the epilogue must match the activation).
-  if (const char *force = getenv("HOM_NVTE_GEMM_KERNEL")) {
-    std::string f(force);
-    const size_t comma = f.find(',');
-    const std::string name = f.substr(0, comma);
-    for (int i = 0; i < gemmKernelCount(); i++)
-      if (name == gemmKernelInfo(i).name && gemmKernelInfo(i).epilogue == epi) {
-        idx = i;
-        pr.splitK = comma == std::string::npos ? 1 : atoi(f.c_str() + comma + 1);
-      }
-  }
-  const int cls = alignmentClass(pr);
-  if (!kernelFits(gemmKernelInfo(idx), cls)) {
-    idx = fallbackKernel(epi, cls);
-    pr.splitK = 1;
-  }
-  return launchGemm(idx, pr, stream());
+  return launchGemm(chooseNvteKernel(&pr, activation), pr, stream());
 }
 
 // The two halves of the layer-norm pair (LayernormGemmRunner.h:17-361).  Both
@@ -444,7 +453,7 @@ Status runLayernormGemm(int64_t rankA, void *dstA, int64_t rankB, void *dstB,
   HOM_CHECK_RET(A.contiguous(), Status::kInvalidArgument,
                 "layernorm-gemm: A must be a contiguous rank-3 tensor");
   _Float16 *tmp = static_cast<_Float16 *>(
-      scratch(kTemp, size_t(rows) * k * sizeof(_Float16), false));
+      libraryScratch(kTemp, size_t(rows) * k * sizeof(_Float16), false));
   if (!tmp && rows * k > 0)
     return Status::kInternal;
   st = launchApplyRowStatsF16(A.data, Var.data, Mean.data, tmp, rows, k,
@@ -513,28 +522,49 @@ bool GemmProfiler::ensure(Buffer &b, int64_t elems) {
 // Protocol of GemmProfiler::profileHelper (lib/NVGPUKernels/GemmProfiler.cu:
 // 81-120): 10 warm-up launches, then batches of 100 between two events until
 // 500 ms have been spent or the kernel is 1.2x slower than the best so far.
-float GemmProfiler::timeKernel(int idx, int splitK, float previousBest) {
+GemmProblem GemmProfiler::problem(bool bIsNK) const {
   GemmProblem pr{};
   pr.A = a_.data;
-  pr.B = b_.data;
+  pr.B = b_.data; // the same scratch values serve as [K, N] and as [N, K]
   pr.C = beta_ != 0.f ? c_.data : nullptr;
   pr.D = c_.data;
   pr.M = M_;
   pr.N = N_;
   pr.K = K_;
   pr.lda = K_;
-  pr.ldb = N_;
+  pr.ldb = bIsNK ? K_ : N_;
   pr.ldc = N_;
   pr.ldd = N_;
   pr.cRowPeriod = M_;
   pr.alpha = alpha_;
   pr.beta = beta_;
-  pr.bIsNK = false;
+  pr.bIsNK = bIsNK;
+  pr.splitK = 1;
+  return pr;
+}
+
+float GemmProfiler::timeKernel(int idx, int splitK, float previousBest,
+                               bool bIsNK) {
+  GemmProblem pr = problem(bIsNK);
   pr.splitK = splitK;
   hipStream_t s = stream();
   if (hipStreamSynchronize(s) != hipSuccess)
     return INFINITY;
-  for (int i = 0; i < 10; i++)
+  // A kernel that cannot implement the problem (leading dimension or operand
+  // too large for its 32-bit offsets, too many tiles, ...) is skipped, as the
+  // reference skips kernels whose can_implement() fails: the first launch runs
+  // with errors recorded silently instead of aborting the compiler process.
+  {
+    const int savedMode = errorMode();
+    setErrorMode(2);
+    const Status probe = launchGemm(idx, pr, s);
+    setErrorMode(savedMode);
+    if (probe != Status::kSuccess) {
+      (void)takeLastError();
+      return INFINITY;
+    }
+  }
+  for (int i = 0; i < 9; i++)
     if (launchGemm(idx, pr, s) != Status::kSuccess)
       return INFINITY;
   float total = 0.f;
@@ -556,17 +586,10 @@ float GemmProfiler::timeKernel(int idx, int splitK, float previousBest) {
   return total / float(iters);
 }
 
-std::tuple<int64_t, int32_t> GemmProfiler::profile() {
-  const auto key = std::make_tuple(M_, N_, K_, activation_);
-  auto it = cache_.find(key);
-  if (it != cache_.end()) {
-    bestTimeMs_ = std::get<2>(it->second);
-    fprintf(stderr, "Cache hit, Idx = %lld, split k factor = %d\n",
-            (long long)std::get<0>(it->second), std::get<1>(it->second));
-    return {std::get<0>(it->second), std::get<1>(it->second)};
-  }
-  if (!ensure(a_, M_ * K_) || !ensure(b_, K_ * N_) || !ensure(c_, M_ * N_))
-    return {-1, 1};
+// Every eligible manifest kernel x split-K factor for one B layout; a
+// candidate has to beat (bestIdx, bestSplit, bestTime) as passed in.
+void GemmProfiler::sweep(bool bIsNK, int64_t *bestIdx, int32_t *bestSplit,
+                         float *bestTime) {
   const Epilogue epi = epilogueFor(activation_, false);
   // Alignment class (the reference walks {8,4,2,1} over M, N, K:
   // lib/NVGPUKernels/GemmProfiler.cu:170-180; here K must be a multiple of 8
@@ -574,10 +597,6 @@ std::tuple<int64_t, int32_t> GemmProfiler::profile() {
   const int cls = K_ % 8 != 0 ? 1 : (N_ % 8 == 0 ? 8 : (N_ % 2 == 0 ? 2 : 1));
   const int maxSplit = std::max(1, std::min<int>(16, int(K_ / 128)));
   const int cus = deviceInfo().computeUnits > 0 ? deviceInfo().computeUnits : 256;
-
-  int64_t bestIdx = -1;
-  int32_t bestSplit = 1;
-  float bestTime = INFINITY;
   for (int idx = 0; idx < gemmKernelCount(); idx++) {
     const GemmKernelInfo &k = gemmKernelInfo(idx);
     if (k.epilogue != epi || !kernelFits(k, cls))
@@ -591,25 +610,60 @@ std::tuple<int64_t, int32_t> GemmProfiler::profile() {
       // only adds reduction traffic; skip those candidates.
       if (s > 1 && tiles * (s - 1) >= int64_t(cus) * 4)
         break;
-      const float t = timeKernel(idx, s, bestTime);
-      if (t < bestTime) {
-        bestTime = t;
-        bestIdx = idx;
-        bestSplit = s;
+      const float t = timeKernel(idx, s, *bestTime, bIsNK);
+      if (t < *bestTime) {
+        *bestTime = t;
+        *bestIdx = idx;
+        *bestSplit = s;
       }
     }
   }
+}
+
+// mode 0: the reference's protocol (GemmProfiler.cu:143-235): the path
+// nvteGemmF16 takes -- B as [N, K], library-selected kernel -- is timed first
+// and is the baseline; the answer is -1 unless a manifest kernel on row-major B
+// beats it (the compiler then emits nvteGemmF16 for that matmul,
+// HOMNVGPUAutotunePass.cpp:90 + HOMNVGPUToFunc.cpp:125-134).
+// mode 1 / 2: best manifest kernel for row-major / [N, K] B, no baseline.
+std::tuple<int64_t, int32_t> GemmProfiler::run(int mode) {
+  const auto key = std::make_tuple(M_, N_, K_, activation_ * 4 + mode);
+  auto it = cache_.find(key);
+  if (it != cache_.end()) {
+    bestTimeMs_ = std::get<2>(it->second);
+    fprintf(stderr, "Cache hit, Idx = %lld, split k factor = %d\n",
+            (long long)std::get<0>(it->second), std::get<1>(it->second));
+    return {std::get<0>(it->second), std::get<1>(it->second)};
+  }
+  if (!ensure(a_, M_ * K_) || !ensure(b_, K_ * N_) || !ensure(c_, M_ * N_))
+    return {-1, 1};
+  int64_t bestIdx = -1;
+  int32_t bestSplit = 1;
+  float bestTime = INFINITY, baseTime = INFINITY;
+  if (mode == 0) {
+    GemmProblem pr = problem(true);
+    const int nvteIdx = chooseNvteKernel(&pr, activation_);
+    if (nvteIdx >= 0)
+      baseTime = bestTime = timeKernel(nvteIdx, pr.splitK, INFINITY, true);
+  }
+  sweep(mode == 2, &bestIdx, &bestSplit, &bestTime);
   bestTimeMs_ = bestTime;
   fprintf(stderr,
           "Profile for %lld %lld %lld act: %lld done. Best kernel %s, best "
-          "split k factor %d, best time %g ms (%.1f TFLOP/s).\n",
+          "split k factor %d, best time %g ms (%.1f TFLOP/s)",
           (long long)M_, (long long)N_, (long long)K_, (long long)activation_,
-          bestIdx >= 0 ? gemmKernelInfo(int(bestIdx)).name : "none", bestSplit,
-          double(bestTime),
+          bestIdx >= 0 ? gemmKernelInfo(int(bestIdx)).name
+                       : (mode == 0 && baseTime < INFINITY ? "nvte" : "none"),
+          bestSplit, double(bestTime),
           2.0 * double(M_) * double(N_) * double(K_) / (double(bestTime) * 1e9));
+  if (mode == 0)
+    fprintf(stderr, ", speedup compared to nvte %g", double(baseTime / bestTime));
+  fprintf(stderr, ".\n");
   cache_[key] = std::make_tuple(bestIdx, bestSplit, bestTime);
   return {bestIdx, bestSplit};
 }
+
+std::tuple<int64_t, int32_t> GemmProfiler::profile() { return run(0); }
 
 std::tuple<int64_t, int32_t> GemmProfiler::profile(int64_t M, int64_t N,
                                                    int64_t K,
@@ -621,7 +675,19 @@ std::tuple<int64_t, int32_t> GemmProfiler::profile(int64_t M, int64_t N,
   activation_ = activation;
   alpha_ = alpha;
   beta_ = beta;
-  return profile();
+  return run(0);
+}
+
+std::tuple<int64_t, int32_t>
+GemmProfiler::profileLayout(int64_t M, int64_t N, int64_t K, int64_t activation,
+                            float alpha, float beta, bool bIsNK) {
+  M_ = M;
+  N_ = N;
+  K_ = K;
+  activation_ = activation;
+  alpha_ = alpha;
+  beta_ = beta;
+  return run(bIsNK ? 2 : 1);
 }
 
 // ------------------------------------------------------------- layer norm --

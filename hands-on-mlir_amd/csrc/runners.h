@@ -50,11 +50,18 @@ public:
   GemmProfiler(const GemmProfiler &) = delete;
   GemmProfiler &operator=(const GemmProfiler &) = delete;
 
-  // (best 0-based manifest index, best split-K)
+  // (best 0-based manifest index, best split-K); index -1 = no manifest kernel
+  // on row-major B beats the [N, K] path of nvteGemmF16 (the reference's
+  // protocol: the compiler then emits nvteGemmF16 for that matmul).
   std::tuple<int64_t, int32_t> profile();
   std::tuple<int64_t, int32_t> profile(int64_t M, int64_t N, int64_t K,
                                        int64_t activation, float alpha,
                                        float beta);
+  // Best manifest kernel for one B layout (row-major, or [N, K] when bIsNK),
+  // without the baseline; what the table generator asks for.
+  std::tuple<int64_t, int32_t> profileLayout(int64_t M, int64_t N, int64_t K,
+                                             int64_t activation, float alpha,
+                                             float beta, bool bIsNK);
   float bestTimeMs() const { return bestTimeMs_; }
 
 private:
@@ -63,7 +70,10 @@ private:
     int64_t capacity = 0; // elements
   };
   bool ensure(Buffer &b, int64_t elems);
-  float timeKernel(int idx, int splitK, float previousBest);
+  GemmProblem problem(bool bIsNK) const;
+  float timeKernel(int idx, int splitK, float previousBest, bool bIsNK);
+  void sweep(bool bIsNK, int64_t *bestIdx, int32_t *bestSplit, float *bestTime);
+  std::tuple<int64_t, int32_t> run(int mode);
 
   int64_t M_, N_, K_, activation_;
   float alpha_, beta_;

@@ -65,7 +65,11 @@ def bert_encoder(layers=12, hidden=768, heads=12, ffn=3072, bs=8, seq=128, vocab
     pos_type = normal16(g, (seq, hidden), 0.02)
     ids = g.integers(0, vocab, size=(bs, seq)).astype(np.int64)
     lens = seq_lengths(g, bs, seq)
+    # masked-LM head: transform dense [H, H]; the decoder is tied to `word` (drawn last so that the
+    # tensors above do not depend on it)
+    w_transform = normal16(g, (hidden, hidden), 0.02)
     return {"weights": weights, "word": word, "pos_type": pos_type, "ids": ids, "lens": lens,
+            "w_transform": w_transform,
             "mask": mask_from_lengths(lens, seq),
             "dims": dict(layers=layers, hidden=hidden, heads=heads, ffn=ffn, bs=bs, seq=seq,
                          vocab=vocab)}

@@ -35,8 +35,9 @@ public:
       : M_(M), N_(N), K_(K), activation_(activation), alpha_(alpha),
         beta_(beta) {}
 
-  /* (0-based manifest index, split-K factor); (-1, 1) when no kernel could be
-   * timed (no GPU, or no kernel with a matching epilogue). */
+  /* (0-based manifest index, split-K factor); index -1 when the nvteGemmF16
+   * path is the fastest, as in the reference (GemmProfiler.cu:155-167,225-235),
+   * or when no kernel could be timed. */
   std::tuple<int64_t, int32_t> profile() {
     return profile(M_, N_, K_, activation_, alpha_, beta_);
   }

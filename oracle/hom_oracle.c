@@ -306,7 +306,8 @@ ORACLE_API void hom_oracle_row_stats(const float *d, float *var, float *mean,
       sq += (double)d[r * n + j] * d[r * n + j];
     }
     const double m = s / (double)n, ms = sq / (double)n;
-    const double rstd = 1.0 / sqrt(ms - m * m + (double)eps);
+    const double v2 = ms - m * m; /* clamped: cancellation on constant rows */
+    const double rstd = 1.0 / sqrt((v2 > 0.0 ? v2 : 0.0) + (double)eps);
     var[r] = (float)rstd;
     mean[r] = (float)(-m * rstd);
   }

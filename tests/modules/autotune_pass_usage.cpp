@@ -33,8 +33,10 @@ int main(int argc, char **argv) {
     profileMatmulImpl(op, 256, 768, 768, 0, 1.0f, 0.0f);
     printf("%lld %d %s\n", (long long)op.kernelName, op.splitK,
            op.kernelName >= 1 ? homGemmManifestName(int32_t(op.kernelName - 1))
-                              : "none");
-    return op.kernelName >= 1 && op.splitK >= 1 ? 0 : 1;
+                              : "nvte");
+    // kernel number 0 = the nvteGemmF16 path won (the lowering then emits
+    // nvteGemmF16, HOMNVGPUToFunc.cpp:125-134)
+    return op.kernelName >= 0 && op.splitK >= 1 ? 0 : 1;
   }
   printf("%d\n", homGemmManifestSize());
   return 0;

@@ -146,7 +146,9 @@ def test_autotune_pass_usage_runs_on_the_gpu(rt, tmp_path):
     res = subprocess.run([exe, "run"], capture_output=True, text=True, timeout=300)
     assert res.returncode == 0, res.stdout + res.stderr
     num, split, name = res.stdout.strip().splitlines()[-1].split()
-    assert 1 <= int(num) <= len(rt.manifest()) and int(split) >= 1 and name.endswith("_linear")
+    assert 0 <= int(num) <= len(rt.manifest()) and int(split) >= 1
+    # 0 = the [N, K] path of nvteGemmF16 was the fastest (the reference's profiler returns -1 then)
+    assert name == "nvte" if int(num) == 0 else name.endswith("_linear")
 
 
 # ---- argument checking: runs without a GPU because every check precedes the

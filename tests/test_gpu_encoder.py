@@ -99,6 +99,48 @@ def test_pinned_gemm_kernels_in_the_graph(gpu, rt, oracle, synth):
         enc.close()
 
 
+def test_captured_split_k_graph_survives_scratch_growth(gpu, rt, synth):
+    """A captured graph has the split-K workspace address baked into its kernel arguments.  When a later
+    call needs a larger workspace the library must not free the old one: the replay has to keep
+    computing the eager result."""
+    import torch
+    bert = importlib.import_module("hands-on-mlir_amd.bert")
+    model = synth.bert_encoder(layers=2, hidden=128, heads=2, ffn=512, bs=3, seq=64, vocab=1000, config=40)
+    number = {n: i + 1 for i, n, _, _ in rt.manifest()}
+    tile = "hom_gfx950_mfma_f16_s32x32x16gemm_f16_64x64_64x2r2_w2x2_nn_align8_linear"
+    enc = bert.BertEncoder(2, 128, 2, 512, 3, 64, 1000, gemm_mode=1, gelu_form="erf")
+    try:
+        enc.load(model)
+        enc.set_inputs(ids=model["ids"], mask=model["mask"])
+        enc.set_gemm_choice("out", number[tile], 2)
+        enc.set_gemm_choice("ffn2", number[tile], 4)
+        enc.forward()
+        eager = enc.output()
+        enc.capture()
+        enc.replay()
+        assert np.array_equal(enc.output(), eager)
+        # a split-K GEMM whose partial tiles (2048 x 2048 x 4 slices x 4 B = 64 MiB) exceed anything
+        # the encoder asked for: the workspace slot is replaced by a larger buffer
+        before = gpu.homScratchGeneration()
+        M = rt.MemRef.from_tensor
+        ta = torch.randn((1, 2048, 512), device="cuda").half()
+        tb = (torch.randn((1, 512, 2048), device="cuda") * 0.05).half()
+        td = torch.zeros((1, 2048, 2048), dtype=torch.float16, device="cuda")
+        gpu.cutlassGemmF16(*M(ta).args(), False, *M(tb).args(), False, *M(td).args(), *M(td).args(),
+                           0, 1.0, 0.0, number[tile], 4)
+        torch.cuda.synchronize()
+        assert gpu.homScratchGeneration() > before, "the workspace did not grow: the test tests nothing"
+        # fill freshly allocated memory so that a dangling workspace would not go unnoticed
+        junk = [torch.full((8 << 20,), float("nan"), dtype=torch.float32, device="cuda") for _ in range(4)]
+        torch.cuda.synchronize()
+        for _ in range(2):
+            enc.replay()
+            assert np.array_equal(enc.output(), eager), "replay after workspace growth differs from eager"
+        del junk
+    finally:
+        enc.close()
+
+
 def test_bert_base_b8_s128(gpu, oracle, synth):
     bert = importlib.import_module("hands-on-mlir_amd.bert")
     model = synth.bert_encoder()

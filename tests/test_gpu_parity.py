@@ -391,6 +391,25 @@ def test_ln_gemm_pair_shapes(gpu, rt, oracle, Mp, N1, K1, N2, beta):
     assert_close(host(out)[0], want, **GEMM_TOL, what="second product")
 
 
+def test_ln_gemm_pair_constant_rows_stay_finite(gpu, rt):
+    """Rows of D that are constant make E[x^2] - E[x]^2 cancel to zero or just below; with BERT's eps of
+    1e-12 an unclamped difference gives NaN statistics that poison the second product."""
+    M = rt.MemRef.from_tensor
+    for (Mp, N1, K1) in [(128, 768, 64), (100, 250, 72)]:   # fused epilogue, separate statistics kernel
+        a = np.full((1, Mp, K1), 0.25, np.float16)
+        b = np.full((1, K1, N1), 0.125, np.float16)
+        a[0, 1::2] = -0.5
+        ta, tb = dev(a), dev(b)
+        d1 = torch.zeros((1, Mp, N1), dtype=torch.float16, device="cuda")
+        var = torch.zeros((1, Mp, 1), dtype=torch.float16, device="cuda")
+        mean = torch.zeros((1, Mp, 1), dtype=torch.float16, device="cuda")
+        gpu.cutlassGemmWithVarMeanF16(*M(ta).args(), *M(tb).args(), *M(d1).args(), *M(d1).args(),
+                                      *M(var).args(), *M(mean).args(), 1.0, 0.0, 0, 1e-12)
+        v, m = host(var).astype(np.float32), host(mean).astype(np.float32)
+        assert not np.isnan(v).any() and not np.isnan(m).any(), (Mp, N1, K1)
+        assert (v > 0).all()
+
+
 # --------------------------------------------------------------- attention --
 def run_attention(gpu, rt, qkv, lens, heads, scale):
     M = rt.MemRef.from_tensor

@@ -112,6 +112,23 @@ def test_gemm_verify_py_matrices(oracle, literals):
     assert np.allclose(mean, (-m * v).numpy(), rtol=1e-4)
 
 
+def test_row_stats_constant_row_is_finite(oracle):
+    """E[x^2] - E[x]^2 of a constant row is zero up to rounding, possibly negative: the clamp keeps
+    var = 1/sqrt(eps) finite for the tiny eps BERT uses, and mean = -x * var."""
+    x = np.full((3, 768), 0.1, np.float32)
+    x[1] = -7.3
+    x[2] = 1000.25
+    var, mean = oracle.row_stats(x, 1e-12)
+    assert np.isfinite(var).all() and np.isfinite(mean).all()
+    assert np.allclose(var, 1e6, rtol=1e-3) or (var > 1e3).all()
+    # a row with spread is untouched by the clamp
+    g = np.random.default_rng(5)
+    y = g.standard_normal((4, 64)).astype(np.float32)
+    v, m = oracle.row_stats(y, 1e-5)
+    assert np.allclose(v, 1 / np.sqrt(y.astype(np.float64).var(-1) + 1e-5), rtol=1e-5)
+    assert np.allclose(m, -y.astype(np.float64).mean(-1) * v, rtol=1e-4, atol=1e-6)
+
+
 def test_gemm_activation_epilogue(oracle):
     g = np.random.default_rng(2)
     A, B = _rand16(g, (8, 32)), _rand16(g, (32, 8), 0.3)
