@@ -14,7 +14,11 @@
 //   -DHOM_LAYERS= -DHOM_HIDDEN= -DHOM_HEADS= -DHOM_FFN= -DHOM_BATCH= -DHOM_SEQ= -DHOM_VOCAB=
 // Constants (allocConstantNVGPUF16(idx), files in $HOM_CONSTANT_DIR):
 //   0 word embeddings [1, V, H]; 1 position+type embeddings [1, S, H];
-//   2 + 4l .. 5 + 4l: Wqkv [1, H, 3H], Wo [1, H, H], W1 [1, H, F], W2 [1, F, H] of layer l.
+//   2 + 4l .. 5 + 4l: Wqkv [1, H, 3H], Wo [1, H, H], W1 [1, H, F], W2 [1, F, H] of layer l;
+//   with -DHOM_LM_HEAD (the masked-LM head of BertForMaskedLM, the graph the
+//   reference's examples/torch/bert/bert.cu runs to logits [b, s, vocab]):
+//   2 + 4L transform dense [1, H, H], 3 + 4L decoder [1, H, V]; forward then
+//   returns the logits instead of the hidden states.
 // -DHOM_GEMM_NUM=n selects a manifest kernel the way the autotune pass bakes one
 // in (0: the library chooses); -DHOM_USE_NVTE routes GEMMs to nvteGemmF16 with
 // [1, N, K] weights instead.
@@ -30,8 +34,14 @@ constexpr int B = HOM_BATCH, S = HOM_SEQ, V = HOM_VOCAB;
 #ifndef HOM_GEMM_NUM
 #define HOM_GEMM_NUM 0
 #endif
-constexpr int kConstants = 2 + 4 * L;
-constexpr int kManaged = kConstants + 6; // + cu, emb, h, qkv, attn, ffn
+#ifdef HOM_LM_HEAD
+constexpr int kHead = 1;
+#else
+constexpr int kHead = 0;
+#endif
+constexpr int kConstants = 2 + 4 * L + 2 * kHead;
+// + cu, emb, h, qkv, attn, ffn (+ transform output, logits)
+constexpr int kManaged = kConstants + 6 + 2 * kHead;
 
 typedef C_UnrankedMemRefType M;
 
@@ -69,10 +79,19 @@ M forward(const M *t, M ids, M mask) {
     gemm(ffn, w[3], h, 0, 1.0f);
     nvteLayernormF16(h.rank, h.descriptor, 1e-12f);
   }
+  const M *result = &h;
+  if (kHead) {
+    const M &wt = t[2 + 4 * L], &wd = t[3 + 4 * L];
+    const M &tr = t[kConstants + 6], &logits = t[kConstants + 7];
+    gemm(h, wt, tr, 1, 0.0f);
+    nvteLayernormF16(tr.rank, tr.descriptor, 1e-12f);
+    gemm(tr, wd, logits, 0, 0.0f);
+    result = &logits;
+  }
   // A returned unranked memref carries a descriptor the caller frees.
   const size_t bytes = sizeof(int64_t) * (3 + 2 * 3);
-  M out{h.rank, std::malloc(bytes)};
-  std::memcpy(out.descriptor, h.descriptor, bytes);
+  M out{result->rank, std::malloc(bytes)};
+  std::memcpy(out.descriptor, result->descriptor, bytes);
   return out;
 }
 } // namespace
@@ -92,6 +111,10 @@ __attribute__((visibility("default"))) void _hom_ciface_forward_initFn(void **sl
   out[kConstants + 3] = alloc3DMemRefNVGPUF16(B, S, 3 * H);
   out[kConstants + 4] = alloc3DMemRefNVGPUF16(B, S, H);
   out[kConstants + 5] = alloc3DMemRefNVGPUF16(B, S, F);
+  if (kHead) {
+    out[kConstants + 6] = alloc3DMemRefNVGPUF16(B, S, H);
+    out[kConstants + 7] = alloc3DMemRefNVGPUF16(B, S, V);
+  }
 }
 
 __attribute__((visibility("default"))) void _hom_ciface_forward(void **slots) {

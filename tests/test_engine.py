@@ -57,6 +57,54 @@ def test_engine_loads_module_and_reports_errors(tmp_path):
 
 
 @pytest.mark.gpu
+def test_compiled_masked_lm_module_through_engine(gpu, rt, oracle, synth, tmp_path, monkeypatch):
+    """The stand-in module with the LM head (-DHOM_LM_HEAD): forward returns logits [b, s, vocab], as the
+    module the reference's examples/torch/bert/bert.cu loads does."""
+    import torch
+    engine = importlib.import_module("hands-on-mlir_amd.engine")
+    weights = importlib.import_module("hands-on-mlir_amd.weights")
+    enc_test = importlib.import_module("test_gpu_encoder")
+    d = dict(DIMS, vocab=1002)
+    model = synth.bert_encoder(config=43, **d)
+    model["lens"][:] = [64, 9, 40]
+    model["mask"] = synth.mask_from_lengths(model["lens"], d["seq"])
+    consts = [model["word"], model["pos_type"]]
+    for w in model["weights"]:
+        consts += [w[k] for k in ("wqkv", "wo", "w1", "w2")]
+    consts += [model["w_transform"], np.ascontiguousarray(model["word"].T)]
+    for i, c in enumerate(consts):
+        weights.write_binary(str(tmp_path), i, c)
+    monkeypatch.setenv("HOM_CONSTANT_DIR", str(tmp_path))
+    monkeypatch.setitem(DIMS, "vocab", 1002)
+    e = engine.Engine(build_module(tmp_path, ("-DHOM_LM_HEAD",)))
+    try:
+        assert e.arg_num("forward") == 2 + 4 * d["layers"] + 2 + 8
+        ids = torch.from_numpy(model["ids"]).cuda()
+        mask = torch.from_numpy(model["mask"].astype(np.int64)).cuda()
+        M = rt.MemRef.from_tensor
+        res = e.invoke("forward", [M(ids), M(mask)])
+        ptr, sizes, strides = rt.read_descriptor(res)
+        assert res.rank == 3 and sizes == [d["bs"], d["seq"], d["vocab"]]
+        out = torch.empty(sizes, dtype=torch.float16, device="cuda")
+        hip = ctypes.CDLL("libamdhip64.so")
+        hip.hipMemcpy.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int]
+        torch.cuda.synchronize()
+        assert hip.hipMemcpy(out.data_ptr(), ptr, out.numel() * 2, 3) == 0
+        logits = out.cpu().numpy()
+        libc = ctypes.CDLL("libc.so.6")
+        libc.free.argtypes = [ctypes.c_void_p]
+        libc.free(res.descriptor)
+        h_or = enc_test.oracle_forward(oracle, model, "erf").astype(np.float16)
+        want = enc_test.lm_head_oracle(oracle, h_or, model, "erf").reshape(d["bs"], d["seq"], d["vocab"])
+        for b, n in enumerate(model["lens"]):
+            err = np.abs(logits[b, :n].astype(np.float64) - want[b, :n])
+            assert (err <= 1e-2 + 1e-3 * np.abs(want[b, :n])).all(), (b, err.max())
+        e.dealloc("forward")
+    finally:
+        e.close()
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("variant", ["manifest", "nvte"])
 def test_compiled_module_through_engine(gpu, rt, oracle, synth, tmp_path, monkeypatch, variant):
     import torch

@@ -33,6 +33,18 @@ def oracle_forward(oracle, model, gelu, round_intermediates=True):
                                round_intermediates=round_intermediates)
 
 
+def lm_head_oracle(oracle, h16, model, gelu, rows=None):
+    """Masked-LM head composed from the pinned oracle pieces, fp16 at every tensor the GPU path stores:
+    t = LN(GELU(h . Wt)), logits = t . word^T (decoder tied to the word embeddings, biases and affine
+    parameters default-initialised, i.e. folded away).  h16: [rows_total, H] fp16; rows: optional row subset."""
+    h = np.ascontiguousarray(h16.reshape(-1, h16.shape[-1]))
+    if rows is not None:
+        h = np.ascontiguousarray(h[rows])
+    t = oracle.gemm(h, model["w_transform"], act="gelu_" + gelu).astype(np.float16)
+    t = oracle.layernorm_f16(t, 1e-12).astype(np.float16)
+    return oracle.gemm(t, model["word"], b_is_nk=True)
+
+
 def check(got, want32, lens, what, rel_limit=1e-3):
     errs, norms = 0.0, 0.0
     for b, n in enumerate(lens):
@@ -71,6 +83,76 @@ def test_small_encoder_eager_and_graph(gpu, oracle, synth, gemm_mode, gelu):
             assert np.array_equal(enc.output(), eager)
     finally:
         enc.close()
+
+
+@pytest.mark.parametrize("gemm_mode,gelu", [(1, "erf"), (0, "tanh")])
+def test_masked_lm_small(gpu, oracle, synth, gemm_mode, gelu):
+    """Encoder + LM head from token ids to logits [b, s, vocab] (vocab 1000: the aligned decoder kernels;
+    vocab 1002: N not a multiple of 8, the 4-byte-row kernels the real 30522 needs)."""
+    bert = importlib.import_module("hands-on-mlir_amd.bert")
+    for vocab in (1000, 1002):
+        model = synth.bert_encoder(layers=2, hidden=128, heads=2, ffn=512, bs=3, seq=64, vocab=vocab, config=40)
+        model["lens"][:] = [64, 17, 33]
+        model["mask"] = synth.mask_from_lengths(model["lens"], 64)
+        enc = bert.BertEncoder(2, 128, 2, 512, 3, 64, vocab, gemm_mode=gemm_mode, gelu_form=gelu, lm_head=True)
+        try:
+            enc.load(model)
+            enc.set_inputs(ids=model["ids"], mask=model["mask"])
+            enc.forward()
+            hidden, logits = enc.output(), enc.logits()
+            # the head alone, from the hidden states the GPU produced: GEMM tolerance
+            want = lm_head_oracle(oracle, hidden, model, gelu).reshape(3, 64, vocab)
+            # the whole graph from token ids against the fp16-faithful oracle chain
+            h_or = oracle_forward(oracle, model, gelu).astype(np.float16)
+            want_chain = lm_head_oracle(oracle, h_or, model, gelu).reshape(3, 64, vocab)
+            for b, n in enumerate(model["lens"]):
+                err = np.abs(logits[b, :n].astype(np.float64) - want[b, :n])
+                assert (err <= 1e-2 + 1e-3 * np.abs(want[b, :n])).all(), (vocab, b, err.max())
+                errc = np.abs(logits[b, :n].astype(np.float64) - want_chain[b, :n])
+                assert (errc <= 1e-2 + 1e-3 * np.abs(want_chain[b, :n])).all(), (vocab, b, errc.max())
+            enc.capture()
+            enc.replay()
+            assert np.array_equal(enc.logits(), logits), "graph replay differs from eager"
+        finally:
+            enc.close()
+
+
+def test_masked_lm_bert_base_b8_s128(gpu, oracle, synth):
+    """BASELINE config 4 with the LM head (the reference's BertForMaskedLM graph, logits [8, 128, 30522]):
+    the head is checked from the GPU's own hidden states on 96 sampled valid positions x all 30522
+    columns (GEMM tolerance rtol 1e-3 / atol 1e-2); the encoder in front of it has its own test."""
+    bert = importlib.import_module("hands-on-mlir_amd.bert")
+    model = synth.bert_encoder()
+    d = model["dims"]
+    enc = bert.BertEncoder(d["layers"], d["hidden"], d["heads"], d["ffn"], d["bs"], d["seq"], d["vocab"],
+                           gemm_mode=1, gelu_form="erf", lm_head=True)
+    try:
+        enc.load(model)
+        enc.set_inputs(ids=model["ids"], mask=model["mask"])
+        enc.capture()
+        enc.replay()
+        hidden, logits = enc.output(), enc.logits()
+    finally:
+        enc.close()
+    assert np.isfinite(logits.astype(np.float32)).all()
+    g = np.random.default_rng(7)
+    rows = []
+    for b, n in enumerate(model["lens"]):
+        rows += [b * d["seq"] + int(s) for s in g.choice(int(n), size=12, replace=False)]
+    rows = np.array(sorted(rows))
+    want = lm_head_oracle(oracle, hidden, model, "erf", rows=rows)
+    got = logits.reshape(-1, d["vocab"])[rows].astype(np.float64)
+    err = np.abs(got - want)
+    assert (err <= 1e-2 + 1e-3 * np.abs(want)).all(), f"LM head: max err {err.max():.3e}"
+    # every one of the 1024 positions through a row checksum: sum_j logits[i, j] = t[i, :] . sum_j word[j, :]
+    # (30522 fp16 roundings of ~1.3e-4 each add up to ~0.03; a wrong tile or a dropped K slab moves a row's sum
+    # by far more than the 0.25 allowed)
+    h_all = np.ascontiguousarray(hidden.reshape(-1, d["hidden"]))
+    t = oracle.layernorm_f16(oracle.gemm(h_all, model["w_transform"], act="gelu_erf").astype(np.float16),
+                             1e-12).astype(np.float16).astype(np.float64)
+    checksum = t @ model["word"].astype(np.float64).sum(0)
+    sums = logits.reshape(-1, d["vocab"]).astype(np.float64).sum(1)
+    assert np.abs(sums - checksum).max() < 0.25, np.abs(sums - checksum).max()
 
 
 def test_pinned_gemm_kernels_in_the_graph(gpu, rt, oracle, synth):
