@@ -117,8 +117,35 @@ inline bool aligned16(const void *p) {
   return (reinterpret_cast<uintptr_t>(p) & 15) == 0;
 }
 
+// Split-K partial tiles of the entry point that may not allocate
+// (homGemmF16NoAlloc): a fixed device array instead of the grow-only buffer.
+// Every GPU the library runs on holds its own copy for the life of the
+// process.  The name below is only a host-side handle; the device address is
+// looked up once per device with hipGetSymbolAddress and kernels get that.
+constexpr size_t kNoAllocScratchBytes = size_t(32) << 20;
+constexpr int kMaxDevices = 64;
+static __device__ __align__(256) unsigned char scratch[kNoAllocScratchBytes];
+void *g_scratchAddress[kMaxDevices] = {};
+
 } // namespace
 
+Status noAllocWorkspace(float **ptr, size_t *bytes) {
+  int dev = -1;
+  HOM_HIP_RET(hipGetDevice(&dev), Status::kInternal);
+  HOM_CHECK_RET(dev >= 0 && dev < kMaxDevices, Status::kInternal,
+                "gemm: device ordinal %d not supported (max %d)", dev,
+                kMaxDevices - 1);
+  if (!g_scratchAddress[dev]) {
+    void *p = nullptr;
+    HOM_HIP_RET(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)), Status::kInternal);
+    HOM_CHECK_RET(p != nullptr, Status::kInternal,
+                  "gemm: no device address for the fixed scratch array");
+    g_scratchAddress[dev] = p;
+  }
+  *ptr = static_cast<float *>(g_scratchAddress[dev]);
+  *bytes = kNoAllocScratchBytes;
+  return Status::kSuccess;
+}
 
 int gemmKernelCount() { return kNumKernels; }
 const GemmKernelInfo &gemmKernelInfo(int idx) { return kKernels[idx].info; }

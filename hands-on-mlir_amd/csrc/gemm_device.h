@@ -474,10 +474,19 @@ Status planLaunch(const GemmProblem &pr, LaunchPlan *plan) {
   if (splitK > 1) {
     const size_t wsBytes =
         size_t(plan->nTiles) * splitK * size_t(BM) * BN * sizeof(float);
-    p.workspace =
-        static_cast<float *>(libraryScratch(kWorkspace, wsBytes, false));
-    if (!p.workspace)
-      return Status::kInternal;
+    if (pr.workspace) {
+      // caller-provided partial-tile buffer: nothing may be allocated here
+      HOM_CHECK_RET(wsBytes <= pr.workspaceBytes, Status::kInvalidArgument,
+                    "gemm: split-K %d of this problem needs %zu bytes of "
+                    "partial tiles, the workspace holds %zu",
+                    splitK, wsBytes, pr.workspaceBytes);
+      p.workspace = pr.workspace;
+    } else {
+      p.workspace =
+          static_cast<float *>(libraryScratch(kWorkspace, wsBytes, false));
+      if (!p.workspace)
+        return Status::kInternal;
+    }
   }
   return Status::kSuccess;
 }

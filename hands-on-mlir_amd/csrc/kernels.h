@@ -76,6 +76,11 @@ struct GemmProblem {
   float alpha, beta;
   bool bIsNK;
   int splitK;
+  // Split-K partial tiles: null = the library's grow-only scratch (allocated
+  // on demand); otherwise a caller-owned device buffer of workspaceBytes that
+  // must be large enough (the launch fails instead of allocating).
+  float *workspace;
+  size_t workspaceBytes;
   // Layer-norm pair, used by launchGemmRowStats / launchGemmRowAffine only
   // (null otherwise).
   // Out: (sum, sum of squares) of every stored row piece, one float2 per row
@@ -109,6 +114,9 @@ int gemmKernelCount();
 const GemmKernelInfo &gemmKernelInfo(int idx);
 // Validates alignment/split-K against the kernel and launches it.
 Status launchGemm(int idx, const GemmProblem &p, hipStream_t s);
+// Device address and size of the fixed split-K scratch array of the current
+// device (looked up on the first call per device; never allocates).
+Status noAllocWorkspace(float **ptr, size_t *bytes);
 
 // The layer-norm pair with the normalisation folded into the two GEMMs'
 // epilogues.  Both need the vector alignment class (K, N and the leading

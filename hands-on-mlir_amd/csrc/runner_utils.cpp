@@ -52,6 +52,17 @@ void cutlassGemmF16(int64_t rankA, void *dstA, bool transa, int64_t rankB,
                         activation, alpha, beta, gemmNum, splitKFactor);
 }
 
+void homGemmF16NoAlloc(int64_t rankA, void *dstA, bool transa, int64_t rankB,
+                       void *dstB, bool transb, int64_t rankC, void *dstC,
+                       int64_t rankD, void *dstD, int64_t activation,
+                       float alpha, float beta, int32_t gemmNum,
+                       int32_t splitKFactor) {
+  (void)transa;
+  (void)transb;
+  (void)runGemmManifest(rankA, dstA, rankB, dstB, rankC, dstC, rankD, dstD,
+                        activation, alpha, beta, gemmNum, splitKFactor, true);
+}
+
 void nvteGemmF16(int64_t rankA, void *dstA, bool transa, int64_t rankB,
                  void *dstB, bool transb, int64_t rankC, void *dstC,
                  int64_t rankD, void *dstD, int64_t activation, float alpha,

@@ -283,13 +283,20 @@ bool selectGemm(int64_t M, int64_t N, int64_t K, int64_t activation,
 Status runGemmManifest(int64_t rankA, void *dstA, int64_t rankB, void *dstB,
                        int64_t rankC, void *dstC, int64_t rankD, void *dstD,
                        int64_t activation, float alpha, float beta,
-                       int32_t gemmNum, int32_t splitK) {
+                       int32_t gemmNum, int32_t splitK, bool noAlloc) {
   View<_Float16> A(rankA, dstA), B(rankB, dstB), C(rankC, dstC), D(rankD, dstD);
   GemmProblem pr{};
   GemmShapes sh{};
   Status st = checkGemmOperands(A, B, C, D, false, beta, &sh, &pr);
   if (st != Status::kSuccess)
     return st;
+  if (noAlloc) {
+    // split-K partial tiles go to the fixed device array; a problem that needs
+    // more than it holds is rejected by the launch instead of allocating
+    st = noAllocWorkspace(&pr.workspace, &pr.workspaceBytes);
+    if (st != Status::kSuccess)
+      return st;
+  }
   pr.alpha = alpha;
   pr.beta = beta;
   int idx;

@@ -18,7 +18,7 @@ namespace hom {
 Status runGemmManifest(int64_t rankA, void *dstA, int64_t rankB, void *dstB,
                        int64_t rankC, void *dstC, int64_t rankD, void *dstD,
                        int64_t activation, float alpha, float beta,
-                       int32_t gemmNum, int32_t splitK);
+                       int32_t gemmNum, int32_t splitK, bool noAlloc = false);
 Status runGemmNvte(int64_t rankA, void *dstA, bool transa, int64_t rankB,
                    void *dstB, bool transb, int64_t rankC, void *dstC,
                    int64_t rankD, void *dstD, int64_t activation, float alpha,
