@@ -403,8 +403,8 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(GemmParams p) {
   }
   static_assert(WM * WN * 32 * (WTN * 4 + 16) <= 2 * STAGE_BYTES,
                 "epilogue strips must fit the main loop's LDS");
-  epilogueStoreLds<MI, NI, WTM, WTN, EPI>(p, acc, m0, n0, waveM, waveN, lane,
-                                          wave, smem);
+  epilogueAuto<MI, NI, WTM, WTN, EPI>(p, acc, m0, n0, waveM, waveN, lane, wave,
+                                      smem);
   } // tiles of this workgroup
 }
 
