@@ -9,13 +9,20 @@ from . import hom_runtime as rt
 
 
 class BertEncoder:
+    ROLES = ("qkv", "out", "ffn1", "ffn2", "transform", "decoder")
+
     def __init__(self, layers, hidden, heads, ffn, bs, seq, vocab, gemm_mode=1, gelu_form="erf",
-                 lm_head=False):
+                 lm_head=False, role_layout=None):
+        """role_layout: optional {role: "kn" | "nk"} pinning the weight layout (and with it the entry
+        point: cutlassGemmF16 / nvteGemmF16) of individual GEMM roles; others are decided by the driver."""
         self.drv = rt.load_driver()
         self.dims = dict(layers=layers, hidden=hidden, heads=heads, ffn=ffn, bs=bs, seq=seq, vocab=vocab)
         self.gemm_mode = gemm_mode
-        self.h = self.drv.homBertCreate(layers, hidden, heads, ffn, bs, seq, vocab, gemm_mode,
-                                        1 if gelu_form == "tanh" else 0)
+        layout = (ctypes.c_int32 * 6)(*[-1] * 6)
+        for role, lay in (role_layout or {}).items():
+            layout[self.ROLES.index(role)] = {"kn": 0, "nk": 1}[lay]
+        self.h = self.drv.homBertCreateWithLayout(layers, hidden, heads, ffn, bs, seq, vocab, gemm_mode,
+                                                  1 if gelu_form == "tanh" else 0, layout)
         assert self.h, "homBertCreate failed"
         self.lm_head = lm_head
         if lm_head:
@@ -35,17 +42,17 @@ class BertEncoder:
         """model: dict from synth.bert_encoder().  Weights are [K, N]; the nvte
         path wants them as [N, K], which the compiler would transpose at compile
         time (HOMNVGPULegalizeGemmPass)."""
-        tr = (lambda w: w.T) if self.gemm_mode == 0 else (lambda w: w)
+        nk = [bool(self.drv.homBertRoleIsNK(self.h, r)) for r in range(6)]
         for l, w in enumerate(model["weights"]):
             for which, key in enumerate(("wqkv", "wo", "w1", "w2")):
-                self._upload(l, which, tr(w[key]))
+                self._upload(l, which, w[key].T if nk[which] else w[key])
         self._upload(0, 4, model["word"])
         self._upload(0, 5, model["pos_type"])
         if self.lm_head:
             # the decoder is tied to the word embeddings (BertForMaskedLM): logits = t . word^T, so the
             # [K, N] operand of the manifest path is word^T and the [N, K] operand of the nvte path is word
-            self._upload(0, 6, tr(model["w_transform"]))
-            self._upload(0, 7, model["word"] if self.gemm_mode == 0 else model["word"].T)
+            self._upload(0, 6, model["w_transform"].T if nk[4] else model["w_transform"])
+            self._upload(0, 7, model["word"] if nk[5] else model["word"].T)
 
     def set_inputs(self, ids=None, mask=None, hidden=None):
         p = lambda a, dt: (np.ascontiguousarray(a, dt).ctypes.data_as(ctypes.c_void_p)
@@ -86,6 +93,9 @@ class BertEncoder:
         idx = ("qkv", "out", "ffn1", "ffn2").index(role)
         if self.drv.homBertSetGemmChoice(self.h, idx, gemm_num, split_k) != 0:
             raise ValueError(f"bad kernel choice {gemm_num}/{split_k} for {role}")
+
+    def role_is_nk(self, role):
+        return bool(self.drv.homBertRoleIsNK(self.h, self.ROLES.index(role)))
 
     def gemm_choices(self):
         buf = (ctypes.c_int32 * 8)()

@@ -50,9 +50,14 @@ struct LayerWeights {
   Tensor wqkv, wo, w1, w2; // [1,K,N] (manifest path) or [1,N,K] (nvte path)
 };
 
+// How one GEMM role of the graph is called.  nk: the weight is stored as
+// [1, N, K] and the call goes to nvteGemmF16 -- what the reference's compiler
+// emits for a matmul whose autotune result was "nvte" (kernel number 0);
+// otherwise cutlassGemmF16 with the manifest kernel gemmNum.
 struct GemmChoice {
   int32_t gemmNum = 0; // 1-based manifest index, 0 = library picks
   int32_t splitK = 1;
+  bool nk = false;
 };
 
 } // namespace
@@ -73,6 +78,7 @@ struct HomBertEncoder {
   // masked-LM head (homBertEnableLmHead): transform weight [1,H,H], decoder
   // weight [1,H,V] ([1,H,H] / [1,V,H] on the nvte path), transform output and
   // logits
+  int32_t roleLayout[6] = {-1, -1, -1, -1, -1, -1};
   bool lmHead = false;
   Tensor wTransform, wDecoder, t, logits;
   GemmChoice cQkv, cOut, cFfn1, cFfn2, cTransform, cDecoder;
@@ -116,7 +122,8 @@ Tensor allocI64_2D(int64_t a, int64_t b) {
 
 void gemm(HomBertEncoder *e, const Tensor &a, const Tensor &w, const Tensor &c,
           const Tensor &d, int64_t act, float beta, const GemmChoice &ch) {
-  if (e->gemmMode == 0) {
+  (void)e;
+  if (ch.nk) {
     nvteGemmF16(a.m.rank, a.m.descriptor, false, w.m.rank, w.m.descriptor, true,
                 c.m.rank, c.m.descriptor, d.m.rank, d.m.descriptor, act, 1.0f,
                 beta, 0, 1);
@@ -127,16 +134,32 @@ void gemm(HomBertEncoder *e, const Tensor &a, const Tensor &w, const Tensor &c,
   }
 }
 
+// layout: 0 row-major weight, 1 [N, K] weight, -1 decide here (gemmMode 0: always
+// [N, K]; 1: what the shipped table prefers; 2: what the live autotuner finds).
+// nvteGemmF16 computes the tanh form of GELU only, so a GELU role of an erf
+// graph stays on the manifest path.
 void chooseGemm(HomBertEncoder *e, int64_t M, int64_t N, int64_t K, int64_t act,
-                float beta, GemmChoice *out) {
+                float beta, int layout, GemmChoice *out) {
+  const bool nkAllowed = act == 0 || e->geluForm == 1 || e->gemmMode == 0;
   int64_t idx = -1;
   int32_t sk = 1;
-  if (e->gemmMode == 2)
+  out->nk = false;
+  if (e->gemmMode == 0 || layout == 1) {
+    out->nk = true;
+  } else if (e->gemmMode == 2) {
     homGemmProfile(M, N, K, act, 1.0f, beta, &idx, &sk, nullptr);
-  else
-    homGemmSelect(M, N, K, act, &idx, &sk);
-  out->gemmNum = int32_t(idx + 1);
-  out->splitK = sk;
+    if (idx < 0 && layout == -1 && nkAllowed)
+      out->nk = true;
+    else if (idx < 0)
+      homGemmProfileLayout(M, N, K, act, 1.0f, beta, 0, &idx, &sk, nullptr);
+  } else {
+    if (layout == -1 && nkAllowed && homGemmPrefersNvte(M, N, K, act))
+      out->nk = true;
+    else
+      homGemmSelect(M, N, K, act, &idx, &sk);
+  }
+  out->gemmNum = out->nk ? 0 : int32_t(idx + 1);
+  out->splitK = out->nk ? 1 : sk;
 }
 
 void callList(HomBertEncoder *e, int fromIds) {
@@ -176,10 +199,14 @@ void callList(HomBertEncoder *e, int fromIds) {
 
 } // namespace
 
-// gemmMode / geluForm as documented on HomBertEncoder.
-DRV_EXPORT HomBertEncoder *homBertCreate(int layers, int hidden, int heads,
-                                         int ffn, int batch, int seq, int vocab,
-                                         int gemmMode, int geluForm) {
+// gemmMode / geluForm as documented on HomBertEncoder.  roleLayout: weight
+// layout per GEMM role (QKV, out-proj, FFN1, FFN2, LM transform, LM decoder):
+// 0 [K, N] + cutlassGemmF16, 1 [N, K] + nvteGemmF16, -1 (or a null pointer) the
+// driver decides, see chooseGemm.
+DRV_EXPORT HomBertEncoder *
+homBertCreateWithLayout(int layers, int hidden, int heads, int ffn, int batch,
+                        int seq, int vocab, int gemmMode, int geluForm,
+                        const int32_t *roleLayout) {
   auto *e = new HomBertEncoder();
   e->layers = layers;
   e->hidden = hidden;
@@ -192,15 +219,24 @@ DRV_EXPORT HomBertEncoder *homBertCreate(int layers, int hidden, int heads,
   e->geluForm = geluForm;
   e->eps = 1e-12f;
   e->w.resize(size_t(layers));
-  const bool nk = gemmMode == 0;
+  for (int r = 0; r < 6; r++)
+    e->roleLayout[r] = roleLayout ? roleLayout[r] : -1;
+  {
+    const int64_t M = int64_t(batch) * seq;
+    const int64_t gelu = geluForm == 1 ? 2 : 1;
+    chooseGemm(e, M, 3 * hidden, hidden, 0, 0.0f, e->roleLayout[0], &e->cQkv);
+    chooseGemm(e, M, hidden, hidden, 0, 1.0f, e->roleLayout[1], &e->cOut);
+    chooseGemm(e, M, ffn, hidden, gelu, 0.0f, e->roleLayout[2], &e->cFfn1);
+    chooseGemm(e, M, hidden, ffn, 0, 1.0f, e->roleLayout[3], &e->cFfn2);
+  }
   for (auto &w : e->w) {
-    w.wqkv.m = nk ? alloc3DMemRefNVGPUF16(1, 3 * hidden, hidden)
-                  : alloc3DMemRefNVGPUF16(1, hidden, 3 * hidden);
+    w.wqkv.m = e->cQkv.nk ? alloc3DMemRefNVGPUF16(1, 3 * hidden, hidden)
+                          : alloc3DMemRefNVGPUF16(1, hidden, 3 * hidden);
     w.wo.m = alloc3DMemRefNVGPUF16(1, hidden, hidden);
-    w.w1.m = nk ? alloc3DMemRefNVGPUF16(1, ffn, hidden)
-                : alloc3DMemRefNVGPUF16(1, hidden, ffn);
-    w.w2.m = nk ? alloc3DMemRefNVGPUF16(1, hidden, ffn)
-                : alloc3DMemRefNVGPUF16(1, ffn, hidden);
+    w.w1.m = e->cFfn1.nk ? alloc3DMemRefNVGPUF16(1, ffn, hidden)
+                         : alloc3DMemRefNVGPUF16(1, hidden, ffn);
+    w.w2.m = e->cFfn2.nk ? alloc3DMemRefNVGPUF16(1, hidden, ffn)
+                         : alloc3DMemRefNVGPUF16(1, ffn, hidden);
   }
   e->wordEmb.m = alloc3DMemRefNVGPUF16(1, vocab, hidden);
   e->posType.m = alloc3DMemRefNVGPUF16(1, seq, hidden);
@@ -217,15 +253,22 @@ DRV_EXPORT HomBertEncoder *homBertCreate(int layers, int hidden, int heads,
       !hipOk(hipEventCreate(&e->evStart), "hipEventCreate") ||
       !hipOk(hipEventCreate(&e->evStop), "hipEventCreate"))
     return e;
-  if (gemmMode != 0) {
-    const int64_t M = int64_t(batch) * seq;
-    const int64_t gelu = geluForm == 1 ? 2 : 1;
-    chooseGemm(e, M, 3 * hidden, hidden, 0, 0.0f, &e->cQkv);
-    chooseGemm(e, M, hidden, hidden, 0, 1.0f, &e->cOut);
-    chooseGemm(e, M, ffn, hidden, gelu, 0.0f, &e->cFfn1);
-    chooseGemm(e, M, hidden, ffn, 0, 1.0f, &e->cFfn2);
-  }
   return e;
+}
+
+DRV_EXPORT HomBertEncoder *homBertCreate(int layers, int hidden, int heads,
+                                         int ffn, int batch, int seq, int vocab,
+                                         int gemmMode, int geluForm) {
+  return homBertCreateWithLayout(layers, hidden, heads, ffn, batch, seq, vocab,
+                                 gemmMode, geluForm, nullptr);
+}
+
+// 1 when the weight of a GEMM role (0 QKV, 1 out-proj, 2 FFN1, 3 FFN2, 4 LM
+// transform, 5 LM decoder) is stored as [N, K]; uploads must match.
+DRV_EXPORT int homBertRoleIsNK(HomBertEncoder *e, int role) {
+  const GemmChoice *c[6] = {&e->cQkv,  &e->cOut,       &e->cFfn1,
+                            &e->cFfn2, &e->cTransform, &e->cDecoder};
+  return role >= 0 && role < 6 && c[role]->nk ? 1 : 0;
 }
 
 // Adds the masked-LM head to the call list: allocates its two weights
@@ -235,21 +278,22 @@ DRV_EXPORT HomBertEncoder *homBertCreate(int layers, int hidden, int heads,
 DRV_EXPORT int homBertEnableLmHead(HomBertEncoder *e) {
   if (e->lmHead)
     return 0;
-  const bool nk = e->gemmMode == 0;
+  {
+    const int64_t M = int64_t(e->batch) * e->seq;
+    chooseGemm(e, M, e->hidden, e->hidden, e->geluForm == 1 ? 2 : 1, 0.0f,
+               e->roleLayout[4], &e->cTransform);
+    chooseGemm(e, M, e->vocab, e->hidden, 0, 0.0f, e->roleLayout[5],
+               &e->cDecoder);
+  }
   e->wTransform.m = alloc3DMemRefNVGPUF16(1, e->hidden, e->hidden);
-  e->wDecoder.m = nk ? alloc3DMemRefNVGPUF16(1, e->vocab, e->hidden)
-                     : alloc3DMemRefNVGPUF16(1, e->hidden, e->vocab);
+  e->wDecoder.m = e->cDecoder.nk
+                      ? alloc3DMemRefNVGPUF16(1, e->vocab, e->hidden)
+                      : alloc3DMemRefNVGPUF16(1, e->hidden, e->vocab);
   e->t.m = alloc3DMemRefNVGPUF16(e->batch, e->seq, e->hidden);
   e->logits.m = alloc3DMemRefNVGPUF16(e->batch, e->seq, e->vocab);
   if (!e->wTransform.data() || !e->wDecoder.data() || !e->t.data() ||
       !e->logits.data())
     return -1;
-  if (e->gemmMode != 0) {
-    const int64_t M = int64_t(e->batch) * e->seq;
-    chooseGemm(e, M, e->hidden, e->hidden, e->geluForm == 1 ? 2 : 1, 0.0f,
-               &e->cTransform);
-    chooseGemm(e, M, e->vocab, e->hidden, 0, 0.0f, &e->cDecoder);
-  }
   e->lmHead = true;
   return 0;
 }
@@ -457,6 +501,8 @@ DRV_EXPORT int homBertSetGemmChoice(HomBertEncoder *e, int role,
   if (role < 0 || role > 3 || gemmNum < 1 || gemmNum > homGemmManifestSize() ||
       splitK < 1)
     return -1;
+  if (c[role]->nk)
+    return -2; // the role's weight is [N, K]: it runs through nvteGemmF16
   c[role]->gemmNum = gemmNum;
   c[role]->splitK = splitK;
   return 0;

@@ -271,4 +271,8 @@ int32_t homGemmSelect(int64_t M, int64_t N, int64_t K, int64_t activation,
   return tuned ? 1 : 0;
 }
 
+int32_t homGemmPrefersNvte(int64_t M, int64_t N, int64_t K, int64_t activation) {
+  return gemmPrefersNvte(M, N, K, activation) ? 1 : 0;
+}
+
 } // extern "C"

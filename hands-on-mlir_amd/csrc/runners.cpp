@@ -124,8 +124,11 @@ int findKernel(int tileM, int tileN, int tileK, Epilogue epi, int alignment) {
 struct TunedEntry {
   int64_t M, N, K;
   int activation; // 0 linear, 1 gelu erf, 2 gelu tanh
-  const char *kernel;
+  const char *kernel; // best kernel for row-major B ([K, N])
   int splitK;
+  const char *nkKernel; // best kernel for B given as [N, K] (may be null)
+  int nkSplitK;
+  int preferNK; // 1: the [N, K] path (nvteGemmF16) is the faster of the two
 };
 
 // Produced on an MI355X by the autotuner (hands-on-mlir_amd/tune_gemm.py) for
@@ -134,7 +137,27 @@ struct TunedEntry {
 // (python/gemm_generator.py:237-278).
 const TunedEntry kTuned[] = {
 #include "gemm_tuned_table.inc"
-    {0, 0, 0, 0, nullptr, 0}};
+    {0, 0, 0, 0, nullptr, 0, nullptr, 0, 0}};
+
+const TunedEntry *findTuned(int64_t M, int64_t N, int64_t K, int64_t activation) {
+  // HOM_GEMM_IGNORE_TUNED_TABLE=1 answers from the timing model only (to check
+  // the model against the table it was fitted to).
+  static const bool useTable = getenv("HOM_GEMM_IGNORE_TUNED_TABLE") == nullptr;
+  if (!useTable || N % 8 != 0 || K % 8 != 0)
+    return nullptr;
+  for (const TunedEntry *t = kTuned; t->kernel; t++)
+    if (t->M == M && t->N == N && t->K == K && t->activation == activation)
+      return t;
+  return nullptr;
+}
+
+int kernelByName(const char *name) {
+  if (name)
+    for (int i = 0; i < gemmKernelCount(); i++)
+      if (strcmp(gemmKernelInfo(i).name, name) == 0)
+        return i;
+  return -1;
+}
 
 // 8: every operand 16-byte aligned with N, K multiples of 8; 2: K a multiple
 // of 8 and the K-contiguous operands 16-byte aligned, but N (the row length of
@@ -181,23 +204,21 @@ int chooseNvteKernel(GemmProblem *pr, int64_t activation);
 
 } // namespace
 
+bool gemmPrefersNvte(int64_t M, int64_t N, int64_t K, int64_t activation) {
+  const TunedEntry *t = findTuned(M, N, K, activation);
+  return t && t->preferNK && kernelByName(t->nkKernel) >= 0;
+}
+
 bool selectGemm(int64_t M, int64_t N, int64_t K, int64_t activation,
-                int64_t *idx, int32_t *splitK) {
+                int64_t *idx, int32_t *splitK, bool bIsNK) {
   const Epilogue epi = epilogueFor(activation, false);
-  // HOM_GEMM_IGNORE_TUNED_TABLE=1 answers from the timing model only (to check
-  // the model against the table it was fitted to).
-  static const bool useTable = getenv("HOM_GEMM_IGNORE_TUNED_TABLE") == nullptr;
-  if (useTable && N % 8 == 0 && K % 8 == 0) {
-    for (const TunedEntry *t = kTuned; t->kernel; t++) {
-      if (t->M == M && t->N == N && t->K == K && t->activation == activation) {
-        for (int i = 0; i < gemmKernelCount(); i++) {
-          if (strcmp(gemmKernelInfo(i).name, t->kernel) == 0) {
-            *idx = i;
-            *splitK = t->splitK;
-            return true;
-          }
-        }
-      }
+  if (const TunedEntry *t = findTuned(M, N, K, activation)) {
+    const int nk = bIsNK ? kernelByName(t->nkKernel) : -1;
+    const int i = nk >= 0 ? nk : kernelByName(t->kernel);
+    if (i >= 0) {
+      *idx = i;
+      *splitK = nk >= 0 ? t->nkSplitK : t->splitK;
+      return true;
     }
   }
   // Untuned shapes: a timing model of the register-staged kernels, fitted to
@@ -333,7 +354,7 @@ int chooseNvteKernel(GemmProblem *pr, int64_t activation) {
   int32_t sk;
   const Epilogue epi = epilogueFor(activation, true);
   selectGemm(pr->M, pr->N, pr->K, epi == Epilogue::kGeluTanh ? 2 : activation,
-             &sel, &sk);
+             &sel, &sk, true);
   int idx = int(sel);
   pr->splitK = sk;
   // Profiling knob: HOM_NVTE_GEMM_KERNEL="<manifest name>[,<splitK>]" pins the
@@ -574,9 +595,16 @@ float GemmProfiler::timeKernel(int idx, int splitK, float previousBest,
   for (int i = 0; i < 9; i++)
     if (launchGemm(idx, pr, s) != Status::kSuccess)
       return INFINITY;
+  // 500 ms per candidate is the reference's budget; HOM_PROFILE_BUDGET_MS
+  // shortens it for table generation over many shapes.
+  static const float budgetMs = [] {
+    const char *v = getenv("HOM_PROFILE_BUDGET_MS");
+    const float f = v ? float(atof(v)) : 500.f;
+    return f > 1.f ? f : 500.f;
+  }();
   float total = 0.f;
   int64_t iters = 0;
-  while (total < 500.f) {
+  while (total < budgetMs) {
     float batch = 0.f;
     (void)hipEventRecord(start_, s);
     for (int i = 0; i < 100; i++)

@@ -38,7 +38,11 @@ Status runLayernormGemm(int64_t rankA, void *dstA, int64_t rankB, void *dstB,
 // `activation`: 0 linear, 1 GELU (erf), 2 GELU (tanh).  Returns true when the
 // shape was found in the tuned table.
 bool selectGemm(int64_t M, int64_t N, int64_t K, int64_t activation,
-                int64_t *idx, int32_t *splitK);
+                int64_t *idx, int32_t *splitK, bool bIsNK = false);
+// Whether the tuned table says that, for this shape, the [N, K] path of
+// nvteGemmF16 beats every manifest kernel on row-major B (what the reference's
+// profiler reports as index -1).
+bool gemmPrefersNvte(int64_t M, int64_t N, int64_t K, int64_t activation);
 
 // Autotuner with the interface of the reference's GemmProfiler
 // (include/NVGPUKernels/GemmProfiler.h:20-57).

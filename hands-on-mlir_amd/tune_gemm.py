@@ -4,16 +4,19 @@ write csrc/gemm_tuned_table.inc (rebuild the library afterwards).
 This is the MI355X counterpart of the reference's compile-time autotune pass
 (lib/Dialect/HOMNVGPU/HOMNVGPUAutotunePass.cpp:52-92 -> GemmProfiler::profile):
 for every (M, N, K, activation) it times each eligible manifest kernel x
-split-K factor through homGemmProfile and records the winner by NAME, so the
-table survives manifest reordering.
+split-K factor, once with B row-major ([K, N], the cutlassGemmF16 path) and
+once with B as [N, K] (the nvteGemmF16 path), and records both winners by
+NAME, so the table survives manifest growth, plus which of the two paths is
+the faster one (what the reference's profiler reports as index -1 = "nvte").
 
-A second pass re-decides the four GEMMs of the BERT-base b8 x s128 and BERT-large
-b32 x s512 encoders inside the captured encoder graph, where operands arrive
-cold from the previous kernel instead of sitting in L2 as in a timing loop:
-one round of coordinate descent over the register-staged tiles, keeping a
-change only if the whole forward gets faster.
+A second pass re-decides the four GEMMs of the BERT-base b8 x s128 and
+BERT-large b32 x s512 encoders inside the captured encoder graph, where
+operands arrive cold from the previous kernel instead of sitting in L2 as in a
+timing loop: one round of coordinate descent over the register-staged tiles
+and over the two weight layouts, keeping a change only if the whole forward
+gets faster.
 
-    python hands-on-mlir_amd/tune_gemm.py [output.inc]     # needs a GPU
+    HOM_PROFILE_BUDGET_MS=150 python hands-on-mlir_amd/tune_gemm.py [output.inc]     # needs a GPU
 """
 import ctypes
 import importlib
@@ -39,8 +42,27 @@ TILES = [(64, 64, 2, 2, 2), (64, 64, 2, 2, 4), (128, 64, 2, 2, 2), (64, 128, 2, 
          (128, 256, 2, 4, 2), (256, 128, 4, 2, 2), (256, 256, 2, 4, 1)]
 
 
+class Row:
+    """One table row: best kernel per layout and the preferred layout."""
+
+    def __init__(self, nn, nn_sk, nn_us, nk, nk_sk, nk_us):
+        self.nn, self.nn_sk, self.nn_us = nn, nn_sk, nn_us
+        self.nk, self.nk_sk, self.nk_us = nk, nk_sk, nk_us
+        # isolated timing: the [N, K] path has to win by more than the noise
+        self.prefer_nk = nk is not None and nk_us < 0.98 * nn_us
+        self.note = ""
+
+    def line(self, key):
+        M, N, K, act = key
+        nk = f'"{self.nk}"' if self.nk else "nullptr"
+        tf = 2.0 * M * N * K / (self.nn_us * 1e6)
+        return (f'    {{{M}, {N}, {K}, {act}, "{self.nn}", {self.nn_sk}, {nk}, {self.nk_sk}, '
+                f'{1 if self.prefer_nk else 0}}}, // [K,N] {self.nn_us:.2f} us ({tf:.0f} TFLOP/s), '
+                f'[N,K] {self.nk_us:.2f} us{self.note}')
+
+
 def in_graph_pass(rt, table):
-    """table: {(M, N, K, act): [name, splitK, note]}; edited in place."""
+    """table: {(M, N, K, act): Row}; edited in place."""
     synth = importlib.import_module("hands-on-mlir_amd.synth")
     bert = importlib.import_module("hands-on-mlir_amd.bert")
     number = {n: i + 1 for i, n, _, _ in rt.manifest()}
@@ -50,21 +72,28 @@ def in_graph_pass(rt, table):
         d = model["dims"]
         M, H, F = d["bs"] * d["seq"], d["hidden"], d["ffn"]
         shapes = {"qkv": (M, 3 * H, H, 0), "out": (M, H, H, 0), "ffn1": (M, F, H, 1), "ffn2": (M, H, F, 0)}
-        enc = bert.BertEncoder(d["layers"], H, d["heads"], F, d["bs"], d["seq"], d["vocab"], gemm_mode=1,
-                               gelu_form="erf")
-        try:
+        layout = {role: "kn" for role in shapes}
+
+        def build(lay):
+            enc = bert.BertEncoder(d["layers"], H, d["heads"], F, d["bs"], d["seq"], d["vocab"], gemm_mode=1,
+                                   gelu_form="erf", role_layout=lay)
             enc.load(model)
             enc.set_inputs(ids=model["ids"], mask=model["mask"])
             for role, key in shapes.items():           # start from the isolated winners
-                if key in table:
-                    enc.set_gemm_choice(role, number[table[key][0]], table[key][1])
+                if key in table and lay[role] == "kn":
+                    enc.set_gemm_choice(role, number[table[key].nn], table[key].nn_sk)
+            return enc
 
-            def forward_us():
-                enc.capture()
-                return min(enc.time(steps, 3, graph=True) for _ in range(3)) * 1e3
+        def forward_us(enc):
+            enc.capture()
+            return min(enc.time(steps, 3, graph=True) for _ in range(3)) * 1e3
+
+        enc = build(layout)
+        try:
+            # tiles of the row-major path, one role at a time
             for role, key in shapes.items():
                 start = enc.gemm_choices()[role]
-                best_us, best = forward_us(), None
+                best_us, best = forward_us(enc), None
                 epi = "gelu" if key[3] == 1 else "linear"
                 for (bm, bn, wm, wn, depth) in TILES:
                     name = (f"hom_gfx950_mfma_f16_s32x32x16gemm_f16_{bm}x{bn}_64x2r{depth}_w{wm}x{wn}"
@@ -72,17 +101,34 @@ def in_graph_pass(rt, table):
                     if number[name] == start[0]:
                         continue
                     enc.set_gemm_choice(role, number[name], 1)
-                    us = forward_us()
+                    us = forward_us(enc)
                     if us < 0.997 * best_us:
                         best_us, best = us, name
                 if best is None:
                     enc.set_gemm_choice(role, *start)
                 else:
                     enc.set_gemm_choice(role, number[best], 1)
-                    table[key] = [best, 1, f"chosen inside the encoder graph ({best_us:.1f} us per forward)"]
+                    table[key].nn, table[key].nn_sk = best, 1
+                    table[key].note = f"; [K,N] tile chosen inside the encoder graph ({best_us:.1f} us per forward)"
                     print(f"in graph: {key} -> {best}", flush=True)
+            base_us = forward_us(enc)
         finally:
             enc.close()
+        # weight layout per role (the erf-GELU role has no [N, K] counterpart: nvteGemmF16 computes tanh)
+        for role, key in shapes.items():
+            if key[3] != 0 or key not in table or table[key].nk is None:
+                continue
+            trial = dict(layout, **{role: "nk"})
+            enc = build(trial)
+            try:
+                us = forward_us(enc)
+            finally:
+                enc.close()
+            table[key].prefer_nk = us < 0.997 * base_us
+            print(f"in graph: {key} [N,K] weights: {us:.1f} us vs {base_us:.1f} us per forward", flush=True)
+            if table[key].prefer_nk:
+                layout, base_us = trial, us
+                table[key].note += f"; [N,K] path chosen inside the encoder graph ({us:.1f} us per forward)"
 
 
 def main():
@@ -92,23 +138,26 @@ def main():
     names = {i: n for i, n, _, _ in rt.manifest()}
     table = {}
     for (M, N, K, act) in bert_shapes():
-        idx, sk, ms = ctypes.c_int64(), ctypes.c_int32(), ctypes.c_float()
         beta = 1.0 if (act == 0 and N in (768, 1024) and K != N // 3) else 0.0
-        lib.homGemmProfile(M, N, K, act, 1.0, beta, ctypes.byref(idx), ctypes.byref(sk), ctypes.byref(ms))
-        if idx.value < 0:
+        res = []
+        for nk in (0, 1):
+            idx, sk, ms = ctypes.c_int64(), ctypes.c_int32(), ctypes.c_float()
+            lib.homGemmProfileLayout(M, N, K, act, 1.0, beta, nk, ctypes.byref(idx), ctypes.byref(sk),
+                                     ctypes.byref(ms))
+            res.append((names.get(idx.value), sk.value, ms.value * 1e3))
+        if res[0][0] is None:
             continue
-        tf = 2.0 * M * N * K / (ms.value * 1e9)
-        table[(M, N, K, act)] = [names[idx.value], sk.value, f"{ms.value * 1e3:.2f} us, {tf:.1f} TFLOP/s"]
-        print((M, N, K, act), table[(M, N, K, act)], flush=True)
+        table[(M, N, K, act)] = Row(*res[0], *res[1])
+        print(table[(M, N, K, act)].line((M, N, K, act)), flush=True)
     if "--no-in-graph" not in sys.argv:
         in_graph_pass(rt, table)
-    lines = [f'    {{{M}, {N}, {K}, {act}, "{v[0]}", {v[1]}}}, // {v[2]}' for (M, N, K, act), v in table.items()]
     args = [a for a in sys.argv[1:] if not a.startswith("--")]
     out = args[0] if args else os.path.join(HERE, "csrc", "gemm_tuned_table.inc")
     with open(out, "w") as f:
-        f.write("// (M, N, K, activation: 0 linear / 1 GELU erf / 2 GELU tanh, kernel name, split-K)\n"
+        f.write("// (M, N, K, activation: 0 linear / 1 GELU erf / 2 GELU tanh, kernel for row-major B, its split-K,\n"
+                "//  kernel for B as [N, K] or nullptr, its split-K, 1 if the [N, K] path is the faster one)\n"
                 "// Written by hands-on-mlir_amd/tune_gemm.py on an MI355X; do not edit by hand.\n")
-        f.write("\n".join(lines) + "\n")
+        f.write("\n".join(row.line(key) for key, row in table.items()) + "\n")
     print("wrote", out)
 
 

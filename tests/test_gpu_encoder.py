@@ -155,6 +155,33 @@ def test_masked_lm_bert_base_b8_s128(gpu, oracle, synth):
     assert np.abs(sums - checksum).max() < 0.25, np.abs(sums - checksum).max()
 
 
+def test_mixed_weight_layouts_per_role(gpu, oracle, synth):
+    """A module may mix the two GEMM entry points: matmuls whose autotune result was "nvte" go to
+    nvteGemmF16 with [N, K] weights, the others to cutlassGemmF16 (HOMNVGPUToFunc.cpp:125-134).  The
+    driver pins the layout per role; every mix must compute the same encoder."""
+    bert = importlib.import_module("hands-on-mlir_amd.bert")
+    model = synth.bert_encoder(layers=2, hidden=128, heads=2, ffn=512, bs=3, seq=64, vocab=1000, config=40)
+    want32 = oracle_forward(oracle, model, "tanh")
+    for lay in ({"qkv": "nk"}, {"out": "nk", "ffn2": "nk"}, {"qkv": "nk", "out": "kn", "ffn1": "nk", "ffn2": "nk"}):
+        enc = bert.BertEncoder(2, 128, 2, 512, 3, 64, 1000, gemm_mode=1, gelu_form="tanh", role_layout=lay)
+        try:
+            for role, want in lay.items():
+                assert enc.role_is_nk(role) == (want == "nk")
+            enc.load(model)
+            enc.set_inputs(ids=model["ids"], mask=model["mask"])
+            enc.forward()
+            eager = enc.output()
+            check(eager, want32, model["lens"], f"layout {lay}")
+            enc.capture()
+            enc.replay()
+            assert np.array_equal(enc.output(), eager)
+            if "out" in lay and lay["out"] == "nk":
+                with pytest.raises(ValueError):     # a [N, K] role has no manifest kernel to pin
+                    enc.set_gemm_choice("out", 1, 1)
+        finally:
+            enc.close()
+
+
 def test_pinned_gemm_kernels_in_the_graph(gpu, rt, oracle, synth):
     """The autotuner's in-graph pass pins one GEMM role at a time to another manifest kernel and
     captures again: every such graph must still compute the encoder."""

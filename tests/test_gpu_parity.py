@@ -306,6 +306,19 @@ def test_gemm_exact_cases(gpu, rt, literals):
     assert np.abs(out.astype(np.float64) - c["expect"]).max() < c["tol"]
 
 
+def test_profiler_layout_sweep_and_table_preference(gpu, rt):
+    """homGemmProfileLayout returns a kernel with the matching epilogue for either layout of B, and
+    homGemmPrefersNvte only says yes for shapes the shipped table holds a [N, K] kernel for."""
+    names = {i: n for i, n, _, _ in rt.manifest()}
+    for nk in (0, 1):
+        idx, sk, ms = ctypes.c_int64(), ctypes.c_int32(), ctypes.c_float()
+        gpu.homGemmProfileLayout(256, 768, 768, 0, 1.0, 0.0, nk, ctypes.byref(idx), ctypes.byref(sk),
+                                 ctypes.byref(ms))
+        assert idx.value >= 0 and names[idx.value].endswith("_linear") and sk.value >= 1 and ms.value > 0
+    assert gpu.homGemmPrefersNvte(7, 24, 40, 0) == 0   # not in the table
+    assert gpu.homGemmPrefersNvte(1024, 768, 768, 0) in (0, 1)
+
+
 def test_nvte_gemm_path(gpu, rt, oracle):
     g = np.random.default_rng(34)
     M = rt.MemRef.from_tensor
