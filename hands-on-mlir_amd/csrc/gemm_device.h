@@ -33,6 +33,7 @@
 
 #include "cross_lane.h"
 #include "kernels.h"
+#include "store_policy.h"
 
 #include <algorithm>
 #include <type_traits>
@@ -192,7 +193,7 @@ __device__ __forceinline__ void epilogueStore(const GemmParams &p,
               v += p.beta * c[e];
             o[e] = _Float16(activate<EPI>(v));
           }
-          *reinterpret_cast<half4 *>(p.D + dRow + n) = o;
+          storeWriteThrough(reinterpret_cast<half4 *>(p.D + dRow + n), o);
         } else {
 #pragma unroll
           for (int e = 0; e < 4; e++) {
@@ -200,7 +201,8 @@ __device__ __forceinline__ void epilogueStore(const GemmParams &p,
               float v = p.alpha * acc[i][j][g * 4 + e];
               if (useC)
                 v += p.beta * float(p.C[cRow + n + e]);
-              p.D[dRow + n + e] = _Float16(activate<EPI>(v));
+              storeWriteThrough(p.D + dRow + n + e,
+                                _Float16(activate<EPI>(v)));
             }
           }
         }
@@ -320,7 +322,7 @@ epilogueStoreLds(const GemmParams &p, float16v (&acc)[MI][NI], int m0, int n0,
             }
         }
         if (vec16) {
-          *reinterpret_cast<half8 *>(dPtr) = o;
+          storeWriteThrough(reinterpret_cast<half8 *>(dPtr), o);
         } else {
 #pragma unroll
           for (int e = 0; e < 8; e += 2)
@@ -328,7 +330,7 @@ epilogueStoreLds(const GemmParams &p, float16v (&acc)[MI][NI], int m0, int n0,
               half2v ov;
               ov[0] = o[e];
               ov[1] = o[e + 1];
-              *reinterpret_cast<half2v *>(dPtr + e) = ov;
+              storeWriteThrough(reinterpret_cast<half2v *>(dPtr + e), ov);
             }
         }
       }
@@ -444,7 +446,7 @@ epilogueFast(const GemmParams &p, float16v (&acc)[MI][NI], int m0, int n0,
       const uint32_t row = uint32_t(i * 32 + r);
       __builtin_amdgcn_raw_buffer_store_b128(
           __builtin_bit_cast(u32x4, o), rsrcD,
-          colOff == kOob ? kOob : row * ldd2 + colOff, 0, 0);
+          colOff == kOob ? kOob : row * ldd2 + colOff, 0, kWriteThroughAux);
     }
   }
 }
