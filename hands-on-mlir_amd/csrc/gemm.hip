@@ -34,6 +34,7 @@ namespace gemmk {
   HOM_EXTERN_EPILOGUES(launchPipe, BM, BN, WM, WN, DIST)
 #define HOM_PIPE_TILE_B HOM_PIPE_TILE_A
 #define HOM_PIPE_TILE_C HOM_PIPE_TILE_A
+#define HOM_PIPE_TILE_D HOM_PIPE_TILE_A
 #define HOM_STAGED_TILE(BM, BN, BK, WM, WN, VEC)                               \
   HOM_EXTERN_STAGED(BM, BN, BK, WM, WN, 0, VEC)                                \
   HOM_EXTERN_STAGED(BM, BN, BK, WM, WN, 1, VEC)                                \
@@ -43,6 +44,7 @@ namespace gemmk {
 #undef HOM_PIPE_TILE_A
 #undef HOM_PIPE_TILE_B
 #undef HOM_PIPE_TILE_C
+#undef HOM_PIPE_TILE_D
 #undef HOM_STAGED_TILE
 } // namespace gemmk
 
@@ -105,6 +107,7 @@ struct KernelEntry {
                        VEC),
 #define HOM_PIPE_TILE_B HOM_PIPE_TILE_A
 #define HOM_PIPE_TILE_C HOM_PIPE_TILE_A
+#define HOM_PIPE_TILE_D HOM_PIPE_TILE_A
 
 // Manifest order is part of the ABI: compiled modules carry indices into it.
 // New entries go at the end of gemm_manifest.inc.

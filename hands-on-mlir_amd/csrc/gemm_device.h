@@ -78,6 +78,15 @@ struct GemmParams {
   float alpha, beta;
   int tilesM, tilesN;
   int kTilesPerSlice;
+  // Tile order, prepared on the host so that a workgroup finds its tile with a
+  // few scalar instructions (tileCoordsFast): tiles per XCD (quotient and
+  // remainder), floor(2^32 / d) for the two divisors of the tile walk, the
+  // number of full groups of kGroupM tile rows and the rows of the last group.
+  int xcdQ, xcdR;
+  uint32_t groupMagic, lastRowsMagic;
+  int fullGroups, lastRows;
+  // epilogueFastMode() evaluated on the host for the whole launch
+  int epiMode;
   // layer-norm pair (kEpiRowStats / kEpiRowAffine kernels only)
   float *rowStatPartials;
   const _Float16 *rowScale;
@@ -154,6 +163,41 @@ __device__ __forceinline__ void tileCoords(int tile, int tilesM, int tilesN,
   *tileN = inGroup / rows;
 }
 
+// n / d for n < 2^32 given m = floor(2^32 / d) (0xffffffff for d == 1): the
+// high product is the quotient or one less.
+__device__ __forceinline__ uint32_t divByMagic(uint32_t n, uint32_t d,
+                                               uint32_t m) {
+  const uint32_t q = __umulhi(n, m);
+  return n - q * d >= d ? q + 1 : q;
+}
+inline uint32_t magicFor(uint32_t d) {
+  return d <= 1 ? 0xffffffffu : uint32_t((uint64_t(1) << 32) / d);
+}
+
+// tileForBlock + tileCoords with the divisions prepared on the host; returns
+// the tile id (what tileCoords maps to the same coordinates).
+__device__ __forceinline__ int tileCoordsFast(const GemmParams &p, int pid,
+                                              int *tileM, int *tileN) {
+  const int xcd = pid & (kNumXcd - 1), loc = pid >> 3;
+  static_assert(kNumXcd == 8, "pid >> 3");
+  const uint32_t tile =
+      uint32_t(xcd * p.xcdQ + (xcd < p.xcdR ? xcd : p.xcdR) + loc);
+  const uint32_t groupSize = uint32_t(kGroupM * p.tilesN);
+  const uint32_t g = divByMagic(tile, groupSize, p.groupMagic);
+  const uint32_t inGroup = tile - g * groupSize;
+  static_assert(kGroupM == 8, "inGroup >> 3");
+  if (int(g) < p.fullGroups) {
+    *tileM = int(g * kGroupM + (inGroup & (kGroupM - 1)));
+    *tileN = int(inGroup >> 3);
+  } else {
+    const uint32_t q =
+        divByMagic(inGroup, uint32_t(p.lastRows), p.lastRowsMagic);
+    *tileM = int(g * kGroupM + inGroup - q * uint32_t(p.lastRows));
+    *tileN = int(q);
+  }
+  return int(tile);
+}
+
 // Accumulator layout shared by every kernel here (transposed 32x32 block):
 // accumulator e of lane l is column 8*(e/4) + 4*(l/32) + e%4, row l%32.
 template <int MI, int NI, int WTM, int WTN, int EPI, int VEC>
@@ -227,10 +271,15 @@ epilogueStoreLds(const GemmParams &p, float16v (&acc)[MI][NI], int m0, int n0,
   constexpr int ROW_B = WTN * 4 + 16;
   constexpr int LPR = WTN / 8;  // lanes per row on the way out
   constexpr int RPP = 64 / LPR; // rows per pass
+  // a row width that does not divide the wavefront (96 columns: 12 lanes per
+  // row) leaves 64 - RPP * LPR lanes without work and a partial last pass
+  constexpr int PASSES = (32 + RPP - 1) / RPP;
+  constexpr bool kEven = RPP * LPR == 64 && PASSES * RPP == 32;
   unsigned char *mine = smem + wave * (32 * ROW_B);
   const int l32 = lane % 32, kb = lane / 32;
   const bool useC = p.beta != 0.f;
   const int rr = lane / LPR, cc = (lane % LPR) * 8;
+  const bool laneActive = kEven || lane < RPP * LPR;
   const int n = n0 + waveN * WTN + cc;
   // 16-byte accesses need rows of C and D that start 16-byte aligned
   const bool vec16 = p.ldd % 8 == 0 && (!useC || p.ldc % 8 == 0);
@@ -265,15 +314,17 @@ epilogueStoreLds(const GemmParams &p, float16v (&acc)[MI][NI], int m0, int n0,
                                      (j * 32 + g * 8 + kb * 4) * 4) = v;
       }
 #pragma unroll
-    for (int pass = 0; pass < 32 / RPP; pass++) {
-      const int r = pass * RPP + rr;
+    for (int pass = 0; pass < PASSES; pass++) {
+      const int rWant = pass * RPP + rr;
+      const bool rowActive = laneActive && (kEven || rWant < 32);
+      const int r = kEven ? rWant : (rWant < 32 ? rWant : 31);
       const float4v lo =
           *reinterpret_cast<const float4v *>(mine + r * ROW_B + cc * 4);
       const float4v hi =
           *reinterpret_cast<const float4v *>(mine + r * ROW_B + cc * 4 + 16);
       const int m = m0 + waveM * WTM + i * 32 + r;
       float rowSum = 0.f, rowSq = 0.f;
-      if (m < p.M && n < p.N) {
+      if (rowActive && m < p.M && n < p.N) {
         const _Float16 *cPtr = p.C + int64_t(m % p.cRowPeriod) * p.ldc + n;
         _Float16 *dPtr = p.D + int64_t(m) * p.ldd + n;
         float c[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
@@ -335,6 +386,8 @@ epilogueStoreLds(const GemmParams &p, float16v (&acc)[MI][NI], int m0, int n0,
         }
       }
       if constexpr (EPI == kEpiRowStats) {
+        static_assert(EPI != kEpiRowStats || kEven,
+                      "row statistics need a power-of-two wave tile width");
         // the LPR lanes of a row hold its WTN columns: one partial per row and
         // wavefront column
         rowSum = sumAcrossLanes<LPR>(rowSum);
@@ -370,11 +423,16 @@ epilogueFast(const GemmParams &p, float16v (&acc)[MI][NI], int m0, int n0,
   constexpr int ROW_B = WTN * 4 + 16;
   constexpr int LPR = WTN / 8;  // lanes per row on the way out
   constexpr int RPP = 64 / LPR; // rows per pass
-  constexpr int PASSES = 32 / RPP;
+  // a row width that does not divide the wavefront (96 columns: 12 lanes per
+  // row) leaves 64 - RPP * LPR lanes without work and a partial last pass;
+  // those lanes and rows get an offset outside the descriptors
+  constexpr int PASSES = (32 + RPP - 1) / RPP;
+  constexpr bool kEven = RPP * LPR == 64 && PASSES * RPP == 32;
   constexpr uint32_t kOob = 0x80000000u;
   unsigned char *mine = smem + wave * (32 * ROW_B);
   const int l32 = lane % 32, kb = lane / 32;
   const int rr = lane / LPR, cc = (lane % LPR) * 8;
+  const bool laneActive = kEven || lane < RPP * LPR;
   const int rowBase = m0 + waveM * WTM;
   const int colBase = n0 + waveN * WTN;
   const int n = colBase + cc;
@@ -386,7 +444,7 @@ epilogueFast(const GemmParams &p, float16v (&acc)[MI][NI], int m0, int n0,
       p.D + int64_t(rowBase) * p.ldd + colBase, 0,
       clampBytes((int64_t(rowsLeft) * p.ldd - colBase) * 2), 0x00020000);
   const uint32_t ldd2 = uint32_t(p.ldd) * 2u, ldc2 = uint32_t(p.ldc) * 2u;
-  const uint32_t colOff = n < p.N ? uint32_t(cc) * 2u : kOob;
+  const uint32_t colOff = n < p.N && laneActive ? uint32_t(cc) * 2u : kOob;
   typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
   // source vectors
   float bias[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
@@ -407,9 +465,10 @@ epilogueFast(const GemmParams &p, float16v (&acc)[MI][NI], int m0, int n0,
 #pragma unroll
       for (int ps = 0; ps < PASSES; ps++) {
         const uint32_t r = uint32_t(i * 32 + ps * RPP + rr);
+        const bool off = colOff == kOob || (!kEven && ps * RPP + rr >= 32);
         cv[i][ps] = __builtin_bit_cast(
             half8, __builtin_amdgcn_raw_buffer_load_b128(
-                       rsrcC, colOff == kOob ? kOob : r * ldc2 + colOff, 0, 0));
+                       rsrcC, off ? kOob : r * ldc2 + colOff, 0, 0));
       }
   }
   __syncthreads();
@@ -428,7 +487,9 @@ epilogueFast(const GemmParams &p, float16v (&acc)[MI][NI], int m0, int n0,
       }
 #pragma unroll
     for (int ps = 0; ps < PASSES; ps++) {
-      const int r = ps * RPP + rr;
+      const int rWant = ps * RPP + rr;
+      const bool off = colOff == kOob || (!kEven && rWant >= 32);
+      const int r = kEven ? rWant : (rWant < 32 ? rWant : 31);
       const float4v lo =
           *reinterpret_cast<const float4v *>(mine + r * ROW_B + cc * 4);
       const float4v hi =
@@ -446,7 +507,7 @@ epilogueFast(const GemmParams &p, float16v (&acc)[MI][NI], int m0, int n0,
       const uint32_t row = uint32_t(i * 32 + r);
       __builtin_amdgcn_raw_buffer_store_b128(
           __builtin_bit_cast(u32x4, o), rsrcD,
-          colOff == kOob ? kOob : row * ldd2 + colOff, 0, kWriteThroughAux);
+          off ? kOob : row * ldd2 + colOff, 0, kWriteThroughAux);
     }
   }
 }
@@ -454,7 +515,8 @@ epilogueFast(const GemmParams &p, float16v (&acc)[MI][NI], int m0, int n0,
 
 // Whether epilogueFast applies (wave-uniform), and with which source mode
 // (0 none, 1 bias row, 2 full matrix); -1 = use epilogueStoreLds.
-__device__ __forceinline__ int epilogueFastMode(const GemmParams &p, int tileM) {
+__host__ __device__ __forceinline__ int epilogueFastMode(const GemmParams &p,
+                                                         int tileM) {
   auto al16 = [](const void *q) {
     return (reinterpret_cast<uintptr_t>(q) & 15) == 0;
   };
@@ -480,7 +542,7 @@ __device__ __forceinline__ void
 epilogueAuto(const GemmParams &p, float16v (&acc)[MI][NI], int m0, int n0,
              int waveM, int waveN, int lane, int wave, unsigned char *smem) {
   if constexpr (EPI <= int(Epilogue::kGeluTanh)) {
-    const int mode = epilogueFastMode(p, WTM);
+    const int mode = p.epiMode;
     if (mode == 0)
       return epilogueFast<MI, NI, WTM, WTN, EPI, 0>(p, acc, m0, n0, waveM, waveN,
                                                     lane, wave, smem);
@@ -568,7 +630,11 @@ __device__ __forceinline__ int swzK(int row, int chunk) {
 }
 // Row-major B tiles: a transposing read touches rows k..k+3 and k+8..k+11, 64
 // bytes of each; 64-byte group g of row k lives at position g ^ f(k).
+// A 96-column tile (rows of 192 bytes, three groups) needs none: rows k..k+3
+// start 192 bytes apart, which already spreads their groups over the banks.
 template <int BN> __device__ __forceinline__ int swzN(int k, int group) {
+  if (BN == 96)
+    return group;
   if (BN == 64)
     return group ^ ((k >> 1) & 1);
   return group ^ (k & 3);
@@ -618,6 +684,14 @@ Status planLaunch(const GemmProblem &pr, LaunchPlan *plan) {
   plan->nTiles = int64_t(p.tilesM) * p.tilesN;
   HOM_CHECK_RET(plan->nTiles < (int64_t(1) << 30), Status::kInvalidArgument,
                 "gemm: too many output tiles (%lld)", (long long)plan->nTiles);
+  p.xcdQ = int(plan->nTiles / kNumXcd);
+  p.xcdR = int(plan->nTiles % kNumXcd);
+  p.groupMagic = magicFor(uint32_t(kGroupM) * uint32_t(p.tilesN));
+  p.fullGroups = p.tilesM / kGroupM;
+  p.lastRows = p.tilesM % kGroupM > 0 ? p.tilesM % kGroupM : kGroupM;
+  p.lastRowsMagic = magicFor(uint32_t(p.lastRows));
+  // (the row range a wavefront addresses with 32-bit offsets is at most BM rows)
+  p.epiMode = epilogueFastMode(p, BM);
   p.workspace = nullptr;
   if (splitK > 1) {
     const size_t wsBytes =

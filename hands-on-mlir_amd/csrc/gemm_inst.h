@@ -16,4 +16,5 @@
 #define HOM_PIPE_TILE_A(...)
 #define HOM_PIPE_TILE_B(...)
 #define HOM_PIPE_TILE_C(...)
+#define HOM_PIPE_TILE_D(...)
 #define HOM_STAGED_TILE(...)

@@ -31,7 +31,11 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(GemmParams p) {
 
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
 
-  const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+  // The wavefront index is the same for every lane; saying so keeps what is
+  // derived from it (the wavefront's rows and columns, the descriptors of its
+  // output rows) in scalar registers.
+  const int tid = threadIdx.x, lane = tid % kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
   const int waveM = wave / WN, waveN = wave % WN;
   const int l32 = lane % 32, kb = lane / 32;
 
@@ -40,13 +44,16 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(GemmParams p) {
   // multiple of the XCD count, so a workgroup's tiles stay in its XCD's
   // contiguous range).  A tile's output stores drain and the next tile's first
   // slabs arrive while other work runs, instead of between two workgroups.
+  // The grid never holds more workgroups than there are tiles, so the first
+  // tile needs no test (a test ahead of everything would make the kernel wait
+  // for two kernel-argument fetches in a row).
   const int nTiles = p.tilesM * p.tilesN;
-  for (int vpid = blockIdx.x; vpid < nTiles; vpid += gridDim.x) {
+  int vpid = blockIdx.x;
+  do {
   if (vpid != int(blockIdx.x))
     __syncthreads(); // the previous tile's epilogue strips live in this LDS
-  const int tile = tileForBlock(nTiles, vpid);
   int tileM, tileN;
-  tileCoords(tile, p.tilesM, p.tilesN, &tileM, &tileN);
+  const int tile = tileCoordsFast(p, vpid, &tileM, &tileN);
   const int m0 = tileM * BM, n0 = tileN * BN;
   const int slice = blockIdx.y, numSlices = gridDim.y;
   const int kTiles = (p.K + BK - 1) / BK;
@@ -58,9 +65,11 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(GemmParams p) {
   // ---- global sources ----
   // Buffer loads from descriptors based at this tile's first row (A) / first
   // row or column block (B): a constant 32-bit byte offset per thread plus a
-  // scalar offset per slab.  Rows / columns past the edge are clamped to the
-  // last valid one: what they fetch only reaches outputs that are never
-  // stored.  Every slab issues the same number of loads and there is no branch
+  // scalar offset per slab.  Rows past the edge (of A, of B given as [N, K])
+  // fall outside the descriptor and read as zero; columns of a row-major B past
+  // the edge read whatever follows in memory (the next row, or zero past the
+  // tensor): what they fetch only reaches outputs that are never stored.
+  // Every slab issues the same number of loads and there is no branch
   // around a load, so the compiler's outstanding-load counts are exact (a
   // branch makes it wait for everything in flight and defeats the pipeline).
   // The main loop walks the slice's FULL slabs only and asks for no range
@@ -90,8 +99,11 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(GemmParams p) {
   // row advances by a multiple of 16 per vector, which leaves both swizzles
   // unchanged (they depend on row bits 0..3 only).
   constexpr int DST_STEP = THREADS * 16;
-  static_assert((THREADS / 8) % 16 == 0 && (THREADS / B_VPR) % 4 == 0 &&
-                    (BN != 64 || (THREADS / B_VPR) % 4 == 0),
+  // (a 96-column row-major B tile is stored without a swizzle: its vectors lie
+  // in LDS in the order of their index)
+  static_assert((THREADS / 8) % 16 == 0 &&
+                    (B_NK || BN == 96 ||
+                     (THREADS % B_VPR == 0 && (THREADS / B_VPR) % 4 == 0)),
                 "vector step must preserve the LDS swizzles");
   int aDst0 = 0, bDst0 = 0;
   int aK[A_PER_T], bK[B_PER_T]; // k position inside the slab
@@ -99,9 +111,8 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(GemmParams p) {
   for (int i = 0; i < A_PER_T; i++) {
     const int v = tid + i * THREADS;
     const int r = v / 8, c = v % 8;
-    const int rr = m0 + r < p.M ? r : p.M - 1 - m0;
     aK[i] = c * 8;
-    aOff[i] = (uint32_t(rr) * uint32_t(p.lda) + c * 8) * 2u;
+    aOff[i] = (uint32_t(r) * uint32_t(p.lda) + c * 8) * 2u;
     if (i == 0)
       aDst0 = r * 128 + swzK(r, c) * 16;
   }
@@ -110,15 +121,13 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(GemmParams p) {
     const int v = tid + i * THREADS;
     const int r = v / B_VPR, c = v % B_VPR;
     if (B_NK) {
-      const int rr = n0 + r < p.N ? r : p.N - 1 - n0;
       bK[i] = c * 8;
-      bOff[i] = (uint32_t(rr) * uint32_t(p.ldb) + c * 8) * 2u;
+      bOff[i] = (uint32_t(r) * uint32_t(p.ldb) + c * 8) * 2u;
       if (i == 0)
         bDst0 = r * 128 + swzK(r, c) * 16;
     } else {
-      const int cc = n0 + c * 8 < p.N ? c * 8 : p.N - 8 - n0;
       bK[i] = r;
-      bOff[i] = (uint32_t(r) * uint32_t(p.ldb) + cc) * 2u;
+      bOff[i] = (uint32_t(r) * uint32_t(p.ldb) + c * 8) * 2u;
       if (i == 0)
         bDst0 = r * B_ROW_BYTES + swzN<BN>(r, c / 4) * 64 + (c % 4) * 16;
     }
@@ -397,15 +406,15 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(GemmParams p) {
     });
   }
 
-  if (numSlices > 1) {
-    storePartial<MI, NI, THREADS>(p, acc, tile, slice, numSlices, tid);
-    continue;
-  }
   static_assert(WM * WN * 32 * (WTN * 4 + 16) <= 2 * STAGE_BYTES,
                 "epilogue strips must fit the main loop's LDS");
-  epilogueAuto<MI, NI, WTM, WTN, EPI>(p, acc, m0, n0, waveM, waveN, lane, wave,
-                                      smem);
-  } // tiles of this workgroup
+  if (numSlices > 1)
+    storePartial<MI, NI, THREADS>(p, acc, tile, slice, numSlices, tid);
+  else
+    epilogueAuto<MI, NI, WTM, WTN, EPI>(p, acc, m0, n0, waveM, waveN, lane,
+                                        wave, smem);
+  vpid += gridDim.x;
+  } while (vpid < nTiles); // tiles of this workgroup
 }
 
 template <int BM, int BN, int WM, int WN, int DIST, int EPI, bool B_NK>
