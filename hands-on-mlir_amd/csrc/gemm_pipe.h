@@ -28,16 +28,18 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(GemmParams p) {
   constexpr int B_ROW_BYTES = B_NK ? 128 : BN * 2;
   constexpr int B_VPR = B_ROW_BYTES / 16; // vectors per LDS row of B
   constexpr int KSTEPS = BK / 16;
+  // Tiles up to 128 x 128 serve problems of a few microseconds, where the way
+  // to the first memory request and back counts as much as the main loop;
+  // larger tiles keep the order that suits their register budget.
+  constexpr bool kLatencyFirst = BM * BN <= 128 * 128;
 
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
 
   // The wavefront index is the same for every lane; saying so keeps what is
   // derived from it (the wavefront's rows and columns, the descriptors of its
   // output rows) in scalar registers.
-  const int tid = threadIdx.x, lane = tid % kWave;
-  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
-  const int waveM = wave / WN, waveN = wave % WN;
-  const int l32 = lane % 32, kb = lane / 32;
+  const int tid0 = threadIdx.x;
+  const int wave0 = __builtin_amdgcn_readfirstlane(tid0 / kWave);
 
   // Persistent over tiles: the grid holds at most as many workgroups as fit on
   // the chip at once and each walks tiles pid, pid + grid, ...  (the grid is a
@@ -52,6 +54,17 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(GemmParams p) {
   do {
   if (vpid != int(blockIdx.x))
     __syncthreads(); // the previous tile's epilogue strips live in this LDS
+  // Small tiles (kLatencyFirst): what the tile loop would let the compiler
+  // compute once, ahead of the first tile's loads (fragment addresses, the
+  // epilogue's descriptors), is tied to these two values, which it must take
+  // as new in every round: a kernel that runs a few microseconds cannot afford
+  // a microsecond of set-up in front of its first memory request.
+  int tid = tid0, wave = wave0;
+  if constexpr (kLatencyFirst)
+    asm volatile("" : "+v"(tid), "+s"(wave));
+  const int lane = tid % kWave;
+  const int waveM = wave / WN, waveN = wave % WN;
+  const int l32 = lane % 32, kb = lane / 32;
   int tileM, tileN;
   const int tile = tileCoordsFast(p, vpid, &tileM, &tileN);
   const int m0 = tileM * BM, n0 = tileN * BN;
@@ -76,7 +89,7 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(GemmParams p) {
   // test per vector: vector instructions in that loop cost matrix-core time.
   // A slab requested past the last full one is replaced by the last full one
   // (it is never used), and a partial last slab (K not a multiple of 64) is
-  // multiplied ahead of the loop by a short unpipelined pass whose loads map
+  // multiplied behind the loop by a short unpipelined pass whose loads map
   // vectors at or past kEnd to an offset outside the descriptor (they read as
   // zero without touching memory).
   constexpr uint32_t kOob = 0x80000000u;
@@ -182,6 +195,17 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(GemmParams p) {
     for (int i = 0; i < B_PER_T; i++)
       *reinterpret_cast<half8 *>(sB + bDst0 + i * DST_STEP) = regB[S][i];
   };
+
+  // The first DIST slabs are requested before anything else is set up.
+  // Small tiles: the first DIST slabs are requested before anything else is
+  // set up.
+  if constexpr (kLatencyFirst) {
+    if (nkFull > 0) {
+      staticFor<DIST>(
+          [&](auto d) { loadGlobal(ktBegin + decltype(d)::value, d); });
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
 
   float16v acc[MI][NI];
 #pragma unroll
@@ -365,10 +389,11 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(GemmParams p) {
       }
     });
   };
-  if (hasTail) {
-    // The partial slab, unpipelined: it is one slab of a ragged problem.
+  // The partial slab of a ragged K, unpipelined: one slab of the whole problem.
+  auto raggedSlab = [&]() {
     using Set0 = std::integral_constant<int, 0>;
     loadGlobalChecked(ktBegin + nkFull, Set0{});
+    __syncthreads(); // no wavefront still reads a full slab from buffer 0
     storeLds(0, Set0{});
     __syncthreads();
 #pragma unroll
@@ -379,11 +404,16 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(GemmParams p) {
         acc[m / NI][m % NI] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
             fb[0][m % NI], fa[0][m / NI], acc[m / NI][m % NI], 0, 0, 0);
     }
-    __syncthreads(); // buffer 0 is rewritten by the first full slab
+    __syncthreads(); // buffer 0 may be rewritten
+  };
+  if constexpr (!kLatencyFirst) {
+    if (hasTail)
+      raggedSlab(); // buffer 0 is rewritten by the first full slab afterwards
   }
   if (nk > 0) {
-    staticFor<DIST>(
-        [&](auto d) { loadGlobal(ktBegin + decltype(d)::value, d); });
+    if constexpr (!kLatencyFirst)
+      staticFor<DIST>(
+          [&](auto d) { loadGlobal(ktBegin + decltype(d)::value, d); });
     storeLds(0, std::integral_constant<int, 0>{});
     loadGlobal(ktBegin + DIST, std::integral_constant<int, 0>{});
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
@@ -404,6 +434,10 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(GemmParams p) {
         slab(i + D, std::integral_constant<int, (D + 1) % DIST>{},
              std::true_type{});
     });
+  }
+  if constexpr (kLatencyFirst) {
+    if (hasTail)
+      raggedSlab(); // behind the full slabs, whose requests went out first
   }
 
   static_assert(WM * WN * 32 * (WTN * 4 + 16) <= 2 * STAGE_BYTES,
