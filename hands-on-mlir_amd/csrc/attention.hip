@@ -73,7 +73,9 @@ __attribute__((amdgpu_waves_per_eu(2, KS == 1 ? 4 : 2))) void bertAttentionKerne
   __shared__ __attribute__((aligned(16))) unsigned char smem[2 * kTileBytes];
   unsigned char *const sK = smem, *const sV = smem + kTileBytes;
 
-  const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+  const int tid = threadIdx.x, lane = tid % kWave;
+  // (the same for every lane: what depends on it stays in scalar registers)
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
   const int l32 = lane % 32, hb = lane / 32;
   const int qg = wave % QG, kh = wave / QG; // query group, key share
   // Workgroup id -> (query tile, head, batch).  Workgroups are dealt to the 8
@@ -82,10 +84,14 @@ __attribute__((amdgpu_waves_per_eu(2, KS == 1 ? 4 : 2))) void bertAttentionKerne
   // the query tiles of one pair, so K/V are fetched into one L2 once instead
   // of once per XCD.  Needs the pair count to be a multiple of 8; the
   // 2-wavefront variant (few workgroups, launch-bound) keeps the plain order.
-  int qTile, pair;
-  {
+  // The key-split variant is launched on a (query tile, head, batch) grid: the
+  // same order of workgroups as a flat id, without the divisions that would
+  // stand between the kernel's entry and its first loads.
+  int qTile, head, b;
+  if (KS == 1) {
     const int id = blockIdx.x;
-    if (KS == 1 && pairs % 8 == 0) {
+    int pair;
+    if (pairs % 8 == 0) {
       const int t = id / 8;
       qTile = t % numQTiles;
       pair = (t / numQTiles) * 8 + id % 8;
@@ -93,10 +99,16 @@ __attribute__((amdgpu_waves_per_eu(2, KS == 1 ? 4 : 2))) void bertAttentionKerne
       qTile = id % numQTiles;
       pair = id / numQTiles;
     }
+    head = pair % heads;
+    b = pair / heads;
+  } else {
+    qTile = blockIdx.x;
+    head = blockIdx.y;
+    b = blockIdx.z;
   }
-  const int head = pair % heads, b = pair / heads;
   const int q0 = qTile * (QG * 32) + qg * 32;
   const int cuLo = cu[b], cuHi = cu[b + 1]; // consumed after the first loads are out
+  __builtin_amdgcn_sched_barrier(0); // requested here, not where they are consumed
 
   const int64_t tokStride = int64_t(3) * heads * kHeadDim;
   const _Float16 *base = qkv + int64_t(b) * seq * tokStride;
@@ -146,8 +158,12 @@ __attribute__((amdgpu_waves_per_eu(2, KS == 1 ? 4 : 2))) void bertAttentionKerne
 
   int len = cuHi - cuLo;
   len = len < 0 ? 0 : (len > seq ? seq : len);
-  // A workgroup whose query rows are all padding has nothing to compute.
-  if (qTile * (QG * 32) >= len) {
+  // A workgroup whose query rows are all padding has nothing to compute.  (Not
+  // in the key-split variant: an early exit ahead of the first use of the
+  // prefetched rows lets the compiler move their loads behind the test, i.e.
+  // behind the arrival of the sequence length.  Such a workgroup walks one
+  // empty chunk there and stores zeros at the end.)
+  if (KS == 1 && qTile * (QG * 32) >= len) {
     const int q = q0 + l32;
     if (q < seq && kh == 0) {
       half4 z;
@@ -194,8 +210,14 @@ __attribute__((amdgpu_waves_per_eu(2, KS == 1 ? 4 : 2))) void bertAttentionKerne
       const_cast<_Float16 *>(vBase), 0, int32_t(uint32_t(len) * rowBytes),
       0x00020000);
 
-  const int numChunks = (len + kChunk - 1) / kChunk; // uniform over the workgroup
-  for (int ch = 0; ch < numChunks; ch++) {
+  // uniform over the workgroup; at least one round in the key-split variant,
+  // whose first chunk is already on its way
+  const int numChunks =
+      KS == 2 && len <= kChunk ? 1 : (len + kChunk - 1) / kChunk;
+  // (at least one round in either variant: a loop that may run zero times
+  // would put a test of the sequence length ahead of the prefetched loads)
+  int ch = 0;
+  do {
     const int key0 = ch * kChunk;
     // keys of this chunk that any wavefront will touch, rounded up to a block
     const int live = (len - key0 < kChunk ? ((len - key0 + 63) / 64) * 64 : kChunk);
@@ -361,7 +383,7 @@ __attribute__((amdgpu_waves_per_eu(2, KS == 1 ? 4 : 2))) void bertAttentionKerne
         }
       }
     }
-  }
+  } while (++ch < numChunks);
 
   // ---- merge the key shares ----
   // Share 1 hands (reference, sum, O) of its rows to share 0 through LDS, in
@@ -459,8 +481,11 @@ Status launchBertAttentionF16(const _Float16 *qkv, const int32_t *cuSeqlens,
         qkv, cuSeqlens, out, int(seq), int(heads), nq, int(pairs), scale);
   } else {
     const int nq = int((seq + 63) / 64);
-    bertAttentionKernel<4, 2><<<dim3((unsigned)(nq * pairs)), dim3(256), 0, s>>>(
-        qkv, cuSeqlens, out, int(seq), int(heads), nq, int(pairs), scale);
+    HOM_CHECK_RET(heads < 65536 && bs < 65536, Status::kInvalidArgument,
+                  "attention: heads and batch size must be below 65536");
+    bertAttentionKernel<4, 2>
+        <<<dim3((unsigned)nq, (unsigned)heads, (unsigned)bs), dim3(256), 0, s>>>(
+            qkv, cuSeqlens, out, int(seq), int(heads), nq, int(pairs), scale);
   }
   HOM_HIP_RET(hipGetLastError(), Status::kInternal);
   return Status::kSuccess;

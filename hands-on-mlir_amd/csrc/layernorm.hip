@@ -29,9 +29,10 @@ template <> struct Vec16<float> {
   typedef float type __attribute__((ext_vector_type(4)));
 };
 
-// One wavefront per row; VPL 16-byte vectors per lane.
-template <typename T, int VPL, bool HAS_RES, bool HAS_AFFINE, bool WT>
-__global__ __launch_bounds__(256) void layernormWaveKernel(
+// One wavefront per row; VPL 16-byte vectors per lane.  The streaming form,
+// for tensors beyond the last-level cache: bandwidth bound, default stores.
+template <typename T, int VPL, bool HAS_RES, bool HAS_AFFINE>
+__global__ __launch_bounds__(256) void layernormStreamKernel(
     const T *x, const T *res,
     const T *__restrict__ gamma, const T *__restrict__ beta, T *out,
     int64_t rows, int hidden, float eps) {
@@ -119,10 +120,108 @@ __global__ __launch_bounds__(256) void layernormWaveKernel(
         for (int j = 0; j < N; j++)
           o[j] = T((v[i][j] - mean) * rstd);
       }
-      if constexpr (WT)
-        storeWriteThrough(&orow[idx], o);
-      else
-        orow[idx] = o;
+      orow[idx] = o;
+    }
+  }
+}
+
+// One wavefront per row; VPL 16-byte vectors per lane.  The form for tensors of
+// a few megabytes, which the next kernel of the stream finds in the last-level
+// cache (results written through, see store_policy.h).
+//
+// The kernel is a chain of memory round trips (arguments, row, result) a few
+// hundred nanoseconds each, so everything it will read is requested at once and
+// nothing stands between the requests: a lane without a vector of its own
+// (768 columns: lanes 32..63 of the second vector) and a wavefront past the
+// last row load a valid address again and mask the values, instead of a branch
+// around the load, which would make the second request wait for the first.
+template <typename T, int VPL, bool HAS_RES, bool HAS_AFFINE>
+__global__ __launch_bounds__(256) void layernormWaveKernel(
+    const T *x, const T *res,
+    const T *__restrict__ gamma, const T *__restrict__ beta, T *out,
+    int64_t rows, int hidden, float eps) {
+  using V = typename Vec16<T>::type;
+  constexpr int N = Vec16<T>::kN;
+  constexpr int kRowsPerBlock = 256 / kWave;
+  const int lane = threadIdx.x & (kWave - 1);
+  // the same for every lane of a wavefront: row addresses stay scalar
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  const int64_t rowWant = int64_t(blockIdx.x) * kRowsPerBlock + wave;
+  const bool rowOk = rowWant < rows;
+  const int64_t row = rowOk ? rowWant : rows - 1;
+  const int nvec = hidden / N;
+  const V *xr = reinterpret_cast<const V *>(x + row * hidden);
+  const V *rr = HAS_RES ? reinterpret_cast<const V *>(res + row * hidden)
+                        : nullptr;
+
+  V raw[VPL];
+  V rawRes[VPL];
+  V g[VPL], b[VPL];
+  const bool hasG = HAS_AFFINE && gamma != nullptr;
+  const bool hasB = HAS_AFFINE && beta != nullptr;
+#pragma unroll
+  for (int i = 0; i < VPL; i++) {
+    const int idx = lane + i * kWave;
+    const int at = idx < nvec ? idx : 0;
+    raw[i] = xr[at];
+    if (HAS_RES)
+      rawRes[i] = rr[at];
+    if (HAS_AFFINE) {
+      // (null gamma / beta: wave-uniform branches, taken by nobody or everybody)
+      if (hasG)
+        g[i] = reinterpret_cast<const V *>(gamma)[at];
+      if (hasB)
+        b[i] = reinterpret_cast<const V *>(beta)[at];
+    }
+  }
+  // every request is out before the first value is touched
+  __builtin_amdgcn_sched_barrier(0);
+  float v[VPL][N];
+  float sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < VPL; i++) {
+    const bool mine = lane + i * kWave < nvec;
+#pragma unroll
+    for (int j = 0; j < N; j++) {
+      float f = float(raw[i][j]);
+      if (HAS_RES)
+        f += float(rawRes[i][j]); // the sum stays in fp32
+      f = mine ? f : 0.f;
+      v[i][j] = f;
+      sum += f;
+    }
+  }
+  const float invH = 1.0f / float(hidden);
+  const float mean = waveSum(sum) * invH;
+  float sq = 0.f;
+#pragma unroll
+  for (int i = 0; i < VPL; i++) {
+    const bool mine = lane + i * kWave < nvec;
+#pragma unroll
+    for (int j = 0; j < N; j++) {
+      const float d = mine ? v[i][j] - mean : 0.f;
+      sq += d * d;
+    }
+  }
+  const float var = waveSum(sq) * invH;
+  const float rstd = 1.0f / sqrtf(var + eps);
+
+  V *orow = reinterpret_cast<V *>(out + row * hidden);
+#pragma unroll
+  for (int i = 0; i < VPL; i++) {
+    const int idx = lane + i * kWave;
+    V o;
+#pragma unroll
+    for (int j = 0; j < N; j++) {
+      float y = (v[i][j] - mean) * rstd;
+      if (hasG)
+        y *= float(g[i][j]);
+      if (hasB)
+        y += float(b[i][j]);
+      o[j] = T(y);
+    }
+    if (rowOk && idx < nvec) {
+      storeWriteThrough(&orow[idx], o);
     }
   }
 }
@@ -182,42 +281,42 @@ __global__ __launch_bounds__(256) void layernormBlockKernel(
 }
 
 // Results that the next kernel of the stream will find in the last-level cache
-// (a few megabytes) are written through, so that no dirty lines wait for the
-// end-of-kernel write-back; streaming-size outputs keep the default policy,
-// which sustains more bandwidth (16384 x 1024: 9.8 us against 10.9 us).
-constexpr int64_t kWriteThroughLimitBytes = int64_t(16) << 20;
+// (a few megabytes) take the latency-oriented kernel with write-through stores;
+// streaming-size tensors take the bandwidth-oriented one (16384 x 1024: 9.8 us
+// against 10.4 us with the other).
+constexpr int64_t kSmallTensorBytes = int64_t(16) << 20;
 
-template <typename T, int VPL, bool WT>
+#define HOM_LN_LAUNCH(KERNEL)                                                  \
+  do {                                                                         \
+    if (res) {                                                                 \
+      if (affine)                                                              \
+        KERNEL<T, VPL, true, true>                                             \
+            <<<grid, block, 0, s>>>(x, res, gamma, beta, out, rows, hidden, eps); \
+      else                                                                     \
+        KERNEL<T, VPL, true, false>                                            \
+            <<<grid, block, 0, s>>>(x, res, gamma, beta, out, rows, hidden, eps); \
+    } else {                                                                   \
+      if (affine)                                                              \
+        KERNEL<T, VPL, false, true>                                            \
+            <<<grid, block, 0, s>>>(x, res, gamma, beta, out, rows, hidden, eps); \
+      else                                                                     \
+        KERNEL<T, VPL, false, false>                                           \
+            <<<grid, block, 0, s>>>(x, res, gamma, beta, out, rows, hidden, eps); \
+    }                                                                          \
+  } while (0)
+
+template <typename T, int VPL>
 void launchWave(const T *x, const T *res, const T *gamma, const T *beta, T *out,
                 int64_t rows, int hidden, float eps, hipStream_t s) {
   const int rowsPerBlock = 256 / kWave;
   dim3 grid((unsigned)((rows + rowsPerBlock - 1) / rowsPerBlock)), block(256);
   const bool affine = gamma || beta;
-  if (res) {
-    if (affine)
-      layernormWaveKernel<T, VPL, true, true, WT>
-          <<<grid, block, 0, s>>>(x, res, gamma, beta, out, rows, hidden, eps);
-    else
-      layernormWaveKernel<T, VPL, true, false, WT>
-          <<<grid, block, 0, s>>>(x, res, gamma, beta, out, rows, hidden, eps);
-  } else {
-    if (affine)
-      layernormWaveKernel<T, VPL, false, true, WT>
-          <<<grid, block, 0, s>>>(x, res, gamma, beta, out, rows, hidden, eps);
-    else
-      layernormWaveKernel<T, VPL, false, false, WT>
-          <<<grid, block, 0, s>>>(x, res, gamma, beta, out, rows, hidden, eps);
-  }
-}
-
-template <typename T, int VPL>
-void launchWave(const T *x, const T *res, const T *gamma, const T *beta, T *out,
-                int64_t rows, int hidden, float eps, hipStream_t s) {
-  if (rows * hidden * int64_t(sizeof(T)) <= kWriteThroughLimitBytes)
-    launchWave<T, VPL, true>(x, res, gamma, beta, out, rows, hidden, eps, s);
+  if (rows * hidden * int64_t(sizeof(T)) <= kSmallTensorBytes)
+    HOM_LN_LAUNCH(layernormWaveKernel);
   else
-    launchWave<T, VPL, false>(x, res, gamma, beta, out, rows, hidden, eps, s);
+    HOM_LN_LAUNCH(layernormStreamKernel);
 }
+#undef HOM_LN_LAUNCH
 
 inline bool aligned16(const void *p) {
   return (reinterpret_cast<uintptr_t>(p) & 15) == 0;

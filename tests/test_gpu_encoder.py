@@ -45,13 +45,19 @@ def lm_head_oracle(oracle, h16, model, gelu, rows=None):
     return oracle.gemm(t, model["word"], b_is_nk=True)
 
 
-def check(got, want32, lens, what, rel_limit=1e-3):
+def check(got, want32, lens, what, rel_limit=1e-3, outlier_frac=0.0):
+    """Elementwise |got - want| <= 1e-2 + 1e-3 |want| on the valid positions plus a norm-wise bound.
+    outlier_frac > 0 (only for comparisons of an fp16-storage pipeline with the fp32 reference over a
+    whole 12-layer stack, where the error is accumulated rounding noise with a tail): that fraction of a
+    sequence's elements may lie outside the elementwise bound, none outside twice the bound."""
     errs, norms = 0.0, 0.0
     for b, n in enumerate(lens):
         g, w = got[b, :n].astype(np.float64), want32[b, :n].astype(np.float64)
         err = np.abs(g - w)
-        bad = err > 1e-2 + 1e-3 * np.abs(w)
-        assert not bad.any(), f"{what}: batch {b}: {bad.sum()} elements off, max {err.max():.3e}"
+        bound = 1e-2 + 1e-3 * np.abs(w)
+        bad = err > bound
+        assert bad.sum() <= np.ceil(outlier_frac * bad.size) and not (err > 2 * bound).any(), \
+            f"{what}: batch {b}: {bad.sum()} of {bad.size} elements off, max {err.max():.3e}"
         errs += (err ** 2).sum()
         norms += (w ** 2).sum()
     rel = np.sqrt(errs / norms)
@@ -272,9 +278,9 @@ def test_bert_base_b8_s128(gpu, oracle, synth):
         # rounding): the GPU path must be as close to it as the fp16-faithful oracle is,
         # i.e. fp16 storage -- which the boundary fixes -- is the only error source.
         pure = oracle_forward(oracle, model, "erf", round_intermediates=False)
-        rel32 = check(got, pure, model["lens"], "BERT-base vs fp32 reference", rel_limit=2e-3)
+        rel32 = check(got, pure, model["lens"], "BERT-base vs fp32 reference", rel_limit=2e-3, outlier_frac=1e-5)
         floor = check(faithful.astype(np.float16), pure, model["lens"], "fp16-faithful oracle vs fp32 reference",
-                      rel_limit=2e-3)
+                      rel_limit=2e-3, outlier_frac=1e-5)
         print(f"BERT-base e2e norm-wise relative error: {rel16:.3e} vs fp16-faithful oracle, "
               f"{rel32:.3e} vs fp32 reference (fp16-storage floor {floor:.3e})")
         assert rel32 <= 1.1 * floor, f"GPU path error {rel32:.3e} exceeds the fp16-storage floor {floor:.3e}"
