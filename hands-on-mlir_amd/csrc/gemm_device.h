@@ -237,7 +237,7 @@ __device__ __forceinline__ void epilogueStore(const GemmParams &p,
               v += p.beta * c[e];
             o[e] = _Float16(activate<EPI>(v));
           }
-          storeWriteThrough(reinterpret_cast<half4 *>(p.D + dRow + n), o);
+          *reinterpret_cast<half4 *>(p.D + dRow + n) = o;
         } else {
 #pragma unroll
           for (int e = 0; e < 4; e++) {
@@ -245,8 +245,7 @@ __device__ __forceinline__ void epilogueStore(const GemmParams &p,
               float v = p.alpha * acc[i][j][g * 4 + e];
               if (useC)
                 v += p.beta * float(p.C[cRow + n + e]);
-              storeWriteThrough(p.D + dRow + n + e,
-                                _Float16(activate<EPI>(v)));
+              p.D[dRow + n + e] = _Float16(activate<EPI>(v));
             }
           }
         }
@@ -381,7 +380,7 @@ epilogueStoreLds(const GemmParams &p, float16v (&acc)[MI][NI], int m0, int n0,
               half2v ov;
               ov[0] = o[e];
               ov[1] = o[e + 1];
-              storeWriteThrough(reinterpret_cast<half2v *>(dPtr + e), ov);
+              *reinterpret_cast<half2v *>(dPtr + e) = ov;
             }
         }
       }

@@ -39,7 +39,7 @@ def bert_shapes():
 
 
 TILES = [(64, 64, 2, 2, 2), (64, 64, 2, 2, 4), (128, 64, 2, 2, 2), (64, 128, 2, 2, 2), (128, 128, 2, 4, 2),
-         (128, 256, 2, 4, 2), (256, 128, 4, 2, 2), (256, 256, 2, 4, 1)]
+         (128, 256, 2, 4, 2), (256, 128, 4, 2, 2), (256, 256, 2, 4, 1), (128, 96, 4, 1, 2), (256, 96, 4, 1, 2)]
 
 
 class Row:
