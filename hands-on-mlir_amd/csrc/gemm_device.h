@@ -80,10 +80,11 @@ struct GemmParams {
   int kTilesPerSlice;
   // Tile order, prepared on the host so that a workgroup finds its tile with a
   // few scalar instructions (tileCoordsFast): tiles per XCD (quotient and
-  // remainder), floor(2^32 / d) for the two divisors of the tile walk, the
-  // number of full groups of kGroupM tile rows and the rows of the last group.
+  // remainder), floor(2^32 / d) for the divisor of the tile walk, the number of
+  // full groups of kGroupM tile rows and the rows of the last group.
   int xcdQ, xcdR;
-  uint32_t groupMagic, lastRowsMagic;
+  uint32_t groupMagic;
+  uint32_t cRowMagic; // floor(2^32 / cRowPeriod)
   int fullGroups, lastRows;
   // epilogueFastMode() evaluated on the host for the whole launch
   int epiMode;
@@ -174,6 +175,13 @@ inline uint32_t magicFor(uint32_t d) {
   return d <= 1 ? 0xffffffffu : uint32_t((uint64_t(1) << 32) / d);
 }
 
+// m % cRowPeriod (the row of a shared source that output row m reads).
+__device__ __forceinline__ int rowInPeriod(const GemmParams &p, int m) {
+  const uint32_t q =
+      divByMagic(uint32_t(m), uint32_t(p.cRowPeriod), p.cRowMagic);
+  return m - int(q) * p.cRowPeriod;
+}
+
 // tileForBlock + tileCoords with the divisions prepared on the host; returns
 // the tile id (what tileCoords maps to the same coordinates).
 __device__ __forceinline__ int tileCoordsFast(const GemmParams &p, int pid,
@@ -190,8 +198,8 @@ __device__ __forceinline__ int tileCoordsFast(const GemmParams &p, int pid,
     *tileM = int(g * kGroupM + (inGroup & (kGroupM - 1)));
     *tileN = int(inGroup >> 3);
   } else {
-    const uint32_t q =
-        divByMagic(inGroup, uint32_t(p.lastRows), p.lastRowsMagic);
+    // (only the workgroups of a last, partial group of tile rows get here)
+    const uint32_t q = inGroup / uint32_t(p.lastRows);
     *tileM = int(g * kGroupM + inGroup - q * uint32_t(p.lastRows));
     *tileN = int(q);
   }
@@ -214,7 +222,7 @@ __device__ __forceinline__ void epilogueStore(const GemmParams &p,
     const int m = m0 + waveM * WTM + i * 32 + l32;
     if (m >= p.M)
       continue;
-    const int64_t cRow = int64_t(m % p.cRowPeriod) * p.ldc;
+    const int64_t cRow = int64_t(rowInPeriod(p, m)) * p.ldc;
     const int64_t dRow = int64_t(m) * p.ldd;
 #pragma unroll
     for (int j = 0; j < NI; j++) {
@@ -324,7 +332,7 @@ epilogueStoreLds(const GemmParams &p, float16v (&acc)[MI][NI], int m0, int n0,
       const int m = m0 + waveM * WTM + i * 32 + r;
       float rowSum = 0.f, rowSq = 0.f;
       if (rowActive && m < p.M && n < p.N) {
-        const _Float16 *cPtr = p.C + int64_t(m % p.cRowPeriod) * p.ldc + n;
+        const _Float16 *cPtr = p.C + int64_t(rowInPeriod(p, m)) * p.ldc + n;
         _Float16 *dPtr = p.D + int64_t(m) * p.ldd + n;
         float c[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
         if (useC) {
@@ -688,7 +696,7 @@ Status planLaunch(const GemmProblem &pr, LaunchPlan *plan) {
   p.groupMagic = magicFor(uint32_t(kGroupM) * uint32_t(p.tilesN));
   p.fullGroups = p.tilesM / kGroupM;
   p.lastRows = p.tilesM % kGroupM > 0 ? p.tilesM % kGroupM : kGroupM;
-  p.lastRowsMagic = magicFor(uint32_t(p.lastRows));
+  p.cRowMagic = magicFor(uint32_t(p.cRowPeriod));
   // (the row range a wavefront addresses with 32-bit offsets is at most BM rows)
   p.epiMode = epilogueFastMode(p, BM);
   p.workspace = nullptr;

@@ -12,8 +12,39 @@ namespace gemmk {
 // The vector memory path into registers sustains several times the bandwidth
 // of the LDS-DMA path on this chip, which matters once a CU streams more than
 // ~16 bytes per clock (large tiles, or several workgroups per CU).
+// What the kernel needs on its way to the first loads travels as leading
+// scalar arguments (14 dwords): the command processor delivers those in scalar
+// registers when the wavefront starts (kernel-argument preload, see the
+// Makefile), so the first requests do not wait for an argument fetch from
+// memory.  `rest` holds the same values again plus everything else; its copies
+// of the leading arguments are never read.
+// tileWalk = xcdR | lastRows << 4 | fullGroups << 8.
 template <int BM, int BN, int WM, int WN, int DIST, int EPI, bool B_NK>
-__global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(GemmParams p) {
+__global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(
+    const _Float16 *argA, const _Float16 *argB, int argM, int argN, int argK,
+    int argLda, int argLdb, int argTilesN, int argXcdQ, uint32_t argTileWalk,
+    uint32_t argGroupMagic, int argKTilesPerSlice, GemmParams rest) {
+  // `rest` is read through the kernel-argument pointer, per tile and behind the
+  // first loads (see below): named here, it would be fetched - and waited for
+  // - ahead of everything.
+  (void)rest;
+  constexpr int kRestOffset = 2 * 8 + 10 * 4; // bytes of the leading arguments
+  static_assert(kRestOffset % alignof(GemmParams) == 0, "argument layout");
+  GemmParams p = {};
+  p.A = argA;
+  p.B = argB;
+  p.M = argM;
+  p.N = argN;
+  p.K = argK;
+  p.lda = argLda;
+  p.ldb = argLdb;
+  p.tilesN = argTilesN;
+  p.xcdQ = argXcdQ;
+  p.xcdR = int(argTileWalk & 15u);
+  p.lastRows = int((argTileWalk >> 4) & 15u);
+  p.fullGroups = int(argTileWalk >> 8);
+  p.groupMagic = argGroupMagic;
+  p.kTilesPerSlice = argKTilesPerSlice;
   static_assert(DIST >= 1, "at least one slab of global loads in flight");
   constexpr int BK = 64;
   constexpr int THREADS = WM * WN * kWave;
@@ -49,8 +80,8 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(GemmParams p) {
   // The grid never holds more workgroups than there are tiles, so the first
   // tile needs no test (a test ahead of everything would make the kernel wait
   // for two kernel-argument fetches in a row).
-  const int nTiles = p.tilesM * p.tilesN;
   int vpid = blockIdx.x;
+  int nTiles;
   do {
   if (vpid != int(blockIdx.x))
     __syncthreads(); // the previous tile's epilogue strips live in this LDS
@@ -206,6 +237,22 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(GemmParams p) {
     }
     __builtin_amdgcn_sched_barrier(0);
   }
+  // Everything else the kernel was given.  The pointer is made opaque so that
+  // these fetches (and what is derived from them: the epilogue's descriptors
+  // and range tests) stay here, behind the first loads, in every round.
+#if defined(__HIP_DEVICE_COMPILE__) // (the host pass only needs the kernel's stub)
+  {
+    typedef const __attribute__((address_space(4))) GemmParams *RestPtr;
+    RestPtr late = (RestPtr)(
+        (const __attribute__((address_space(4))) char *)
+            __builtin_amdgcn_kernarg_segment_ptr() +
+        kRestOffset);
+    if constexpr (kLatencyFirst)
+      asm volatile("" : "+s"(late));
+    p = *late;
+  }
+#endif
+  nTiles = p.tilesM * p.tilesN;
 
   float16v acc[MI][NI];
 #pragma unroll
@@ -491,8 +538,14 @@ Status launchPipe(const GemmProblem &pr, hipStream_t s) {
     gridX = std::max<int64_t>(kNumXcd, resident / plan.splitK / kNumXcd * kNumXcd);
   if (gridX > plan.nTiles)
     gridX = plan.nTiles;
+  const GemmParams &q = plan.p;
+  // (leading dimensions fit 31 bits: checked above)
   kernel<<<dim3((unsigned)gridX, (unsigned)plan.splitK), dim3(WM * WN * kWave),
-           SMEM, s>>>(plan.p);
+           SMEM, s>>>(q.A, q.B, q.M, q.N, q.K, int(q.lda), int(q.ldb), q.tilesN,
+                      q.xcdQ,
+                      uint32_t(q.xcdR) | uint32_t(q.lastRows) << 4 |
+                          uint32_t(q.fullGroups) << 8,
+                      q.groupMagic, q.kTilesPerSlice, q);
   HOM_HIP_RET(hipGetLastError(), Status::kInternal);
   if (plan.splitK > 1)
     return launchReduce<BM, BN, WM, WN, EPI, 8>(plan, s);
