@@ -627,6 +627,86 @@ __global__ __launch_bounds__(WM *WN *kWave) void splitKReduceKernel(
                                             wave / WN, wave % WN, lane);
 }
 
+// The same reduction with one thread per group of four outputs instead of one
+// workgroup per tile: a skinny problem (64 x 1024 in 16 tiles) would otherwise
+// reduce on 16 workgroups, each walking the slices of a whole tile in turn.
+// Thread idx owns float4 number idx of the partial-tile layout (tile, block
+// row i, block column j, quad g, thread of the producing workgroup); it adds
+// the slices in slice order, four loads in flight, and finishes its four
+// consecutive columns of one output row.
+template <int BM, int BN, int WM, int WN, int EPI, int VEC>
+__global__ __launch_bounds__(256) void splitKReduceFlatKernel(GemmParams p,
+                                                              int numSlices) {
+  constexpr int THREADS = WM * WN * kWave;
+  constexpr int WTM = BM / WM, WTN = BN / WN;
+  constexpr int MI = WTM / 32, NI = WTN / 32;
+  constexpr int ACC_V4 = MI * NI * 4;
+  constexpr int PER_TILE = ACC_V4 * THREADS; // float4 per partial tile
+  const int64_t idx = int64_t(blockIdx.x) * 256 + threadIdx.x;
+  const int64_t total = int64_t(p.tilesM) * p.tilesN * PER_TILE;
+  if (idx >= total)
+    return;
+  const int tile = int(idx / PER_TILE);
+  const int rem = int(idx % PER_TILE);
+  const int q = rem / THREADS, t = rem % THREADS;
+  const int i = q / (NI * 4), j = (q / 4) % NI, g = q % 4;
+  const int lane = t % kWave, wave = t / kWave;
+  const int l32 = lane % 32, kb = lane / 32;
+  int tileM, tileN;
+  tileCoords(tile, p.tilesM, p.tilesN, &tileM, &tileN);
+  const float4v *part = reinterpret_cast<const float4v *>(p.workspace) +
+                        int64_t(tile) * numSlices * PER_TILE + rem;
+  float4v acc = {0.f, 0.f, 0.f, 0.f};
+  int sl = 0;
+  for (; sl + 4 <= numSlices; sl += 4) {
+    float4v v[4];
+#pragma unroll
+    for (int u = 0; u < 4; u++)
+      v[u] = part[int64_t(sl + u) * PER_TILE];
+#pragma unroll
+    for (int u = 0; u < 4; u++) // slice order: the sum does not depend on timing
+      acc += v[u];
+  }
+  for (; sl < numSlices; sl++)
+    acc += part[int64_t(sl) * PER_TILE];
+  const int m = tileM * BM + (wave / WN) * WTM + i * 32 + l32;
+  const int n = tileN * BN + (wave % WN) * WTN + j * 32 + g * 8 + kb * 4;
+  if (m >= p.M)
+    return;
+  const bool useC = p.beta != 0.f;
+  const int64_t cRow = int64_t(rowInPeriod(p, m)) * p.ldc;
+  const int64_t dRow = int64_t(m) * p.ldd;
+  const bool quadRows = p.ldd % 4 == 0 && (!useC || p.ldc % 4 == 0);
+  if (VEC == 8 && quadRows && n + 4 <= p.N) {
+    float c[4] = {0.f, 0.f, 0.f, 0.f};
+    if (useC) {
+      const half4 cv = *reinterpret_cast<const half4 *>(p.C + cRow + n);
+#pragma unroll
+      for (int e = 0; e < 4; e++)
+        c[e] = float(cv[e]);
+    }
+    half4 o;
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      float v = p.alpha * acc[e];
+      if (useC)
+        v += p.beta * c[e];
+      o[e] = _Float16(activate<EPI>(v));
+    }
+    *reinterpret_cast<half4 *>(p.D + dRow + n) = o;
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      if (n + e < p.N) {
+        float v = p.alpha * acc[e];
+        if (useC)
+          v += p.beta * float(p.C[cRow + n + e]);
+        p.D[dRow + n + e] = _Float16(activate<EPI>(v));
+      }
+    }
+  }
+}
+
 // ===================================================================== dma ==
 // Swizzles (in units of 16-byte chunks / 64-byte groups inside an LDS row).
 // K-contiguous tiles (A, and B given as [N, K]): rows of 128 bytes = 8 chunks;
@@ -733,6 +813,16 @@ template <typename K> Status allowLds(K kernel, int bytes, bool *done) {
 
 template <int BM, int BN, int WM, int WN, int EPI, int VEC>
 Status launchReduce(const LaunchPlan &plan, hipStream_t s) {
+  // Few tiles: spread the reduction over the chip (one thread per four outputs).
+  constexpr int kPerTile = (BM / 32) * (BN / 32) * 4 * kWave; // float4 per tile
+  if (plan.nTiles < 128) {
+    const int64_t groups = plan.nTiles * kPerTile;
+    splitKReduceFlatKernel<BM, BN, WM, WN, EPI, VEC>
+        <<<dim3((unsigned)((groups + 255) / 256)), dim3(256), 0, s>>>(
+            plan.p, plan.splitK);
+    HOM_HIP_RET(hipGetLastError(), Status::kInternal);
+    return Status::kSuccess;
+  }
   splitKReduceKernel<BM, BN, WM, WN, EPI, VEC>
       <<<dim3((unsigned)plan.nTiles), dim3(WM * WN * kWave), 0, s>>>(
           plan.p, plan.splitK);
