@@ -4,6 +4,7 @@
 // tests/test_abi.py against include/NVGPUKernels/GemmProfiler.h and
 // libhom_amdgpu_runner_utils.so; with "run" as its argument it profiles one
 // shape on the GPU and prints the result.
+#include "NVGPUKernels/GemmManifest.h"
 #include "NVGPUKernels/GemmProfiler.h"
 
 #include <cstdio>
@@ -38,6 +39,20 @@ int main(int argc, char **argv) {
     // nvteGemmF16, HOMNVGPUToFunc.cpp:125-134)
     return op.kernelName >= 0 && op.splitK >= 1 ? 0 : 1;
   }
-  printf("%d\n", homGemmManifestSize());
+  // The manifest object (GemmManifest.h:18-65): size, indexing, the runner's
+  // name / activation queries, as GemmProfiler.cu:181-200 walks it.
+  using namespace mlir::hands_on_mlir::homnvgpu_kernel;
+  int gelu = 0;
+  for (size_t i = 0; i < manifest.size(); i++) {
+    auto op = manifest[int(i)];
+    if (!op.isF16() || manifest.find(op.getName()) != int32_t(i))
+      return 2;
+    if (op.contains("gelu") != (op.getActivation() == 1))
+      return 3;
+    gelu += op.getActivation();
+  }
+  if (gelu == 0 || manifest.getKernel(0).getName() == nullptr)
+    return 4;
+  printf("%d\n", int(manifest.size()));
   return 0;
 }
