@@ -44,17 +44,24 @@ typedef short short4v __attribute__((ext_vector_type(4)));
 typedef short short8v __attribute__((ext_vector_type(8)));
 
 constexpr int kWave = 64;
-constexpr int kHeadDim = 64;
 constexpr int kChunk = 128;                  // keys staged per barrier
-constexpr int kTileBytes = kChunk * 128;     // one K or V chunk in LDS
 
-// chunk c (16 bytes) of K row r lives at position c ^ ((r >> 1) & 7)
-__device__ __forceinline__ int swzK(int row, int chunk) {
-  return chunk ^ ((row >> 1) & 7);
+// Head sizes 64 and 128 (template parameter D).  A K or V row in LDS is D
+// halves: 128 bytes = 8 chunks of 16 bytes = 2 groups of 64 bytes for D = 64,
+// twice that for D = 128.
+//
+// chunk c (16 bytes) of K row r lives at position c ^ ((r >> 1) & 7) (rows of
+// 128 bytes: two consecutive rows cover all banks once) or c ^ (r & 15) (rows
+// of 256 bytes: every row starts at bank 0), so that the 128-bit fragment
+// reads of 16 consecutive rows hit 16 distinct bank groups
+template <int D> __device__ __forceinline__ int swzK(int row, int chunk) {
+  return D == 64 ? chunk ^ ((row >> 1) & 7) : chunk ^ (row & 15);
 }
-// 64-byte group g of V row k lives at position g ^ ((k >> 1) & 1)
-__device__ __forceinline__ int swzV(int k, int group) {
-  return group ^ ((k >> 1) & 1);
+// 64-byte group g of V row k lives at position g ^ ((k >> 1) & 1), or
+// g ^ (k & 3) for rows of 256 bytes: a transposing read touches 64 bytes of
+// each of rows k..k+3
+template <int D> __device__ __forceinline__ int swzV(int k, int group) {
+  return D == 64 ? group ^ ((k >> 1) & 1) : group ^ (k & 3);
 }
 
 // NW wavefronts per workgroup, KS of them share each group of 32 query rows
@@ -62,12 +69,17 @@ __device__ __forceinline__ int swzV(int k, int group) {
 // keys of its own 32 rows; KS = 2: half the serial work per wavefront, for
 // short sequences where there are fewer workgroups than CUs and the key walk
 // of one wavefront is the critical path; the halves are merged through LDS).
-template <int NW, int KS>
+template <int NW, int KS, int D>
 __global__ __launch_bounds__(NW *kWave)
-__attribute__((amdgpu_waves_per_eu(2, KS == 1 ? 4 : 2))) void bertAttentionKernel(
+__attribute__((amdgpu_waves_per_eu(D == 64 ? 2 : 1, D == 64 && KS == 1 ? 4 : 2))) void bertAttentionKernel(
     const _Float16 *__restrict__ qkv, const int32_t *__restrict__ cu,
     _Float16 *__restrict__ out, int seq, int heads, int numQTiles, int pairs,
     float scale) {
+  static_assert(D == 64 || D == 128, "head size");
+  constexpr int kHeadDim = D;
+  constexpr int kRowB = D * 2;               // bytes of a K or V row
+  constexpr int CPR = D / 8;                 // 16-byte chunks per row
+  constexpr int kTileBytes = kChunk * kRowB; // one K or V chunk in LDS
   constexpr int kThreads = NW * kWave;
   constexpr int QG = NW / KS; // groups of 32 query rows per workgroup
   __shared__ __attribute__((aligned(16))) unsigned char smem[2 * kTileBytes];
@@ -128,14 +140,15 @@ __attribute__((amdgpu_waves_per_eu(2, KS == 1 ? 4 : 2))) void bertAttentionKerne
   // are wasted on all-padding workgroups, and prefetching the next chunk into
   // registers measured 3-8 % slower than loading each chunk when it is due
   // (also with barriers that do not wait for the prefetch).
-  constexpr bool kPrefetch = KS == 2;
-  constexpr int VPT = kChunk * 8 / kThreads; // vectors of K (and of V) per thread
+  // (D = 128: the prefetched rows would take 64 more registers than there are)
+  constexpr bool kPrefetch = KS == 2 && D == 64;
+  constexpr int VPT = kChunk * CPR / kThreads; // vectors of K (and of V) per thread
   half8 rk[VPT], rv[VPT];
   auto loadChunk = [&](int key0) {
 #pragma unroll
     for (int i = 0; i < VPT; i++) {
       const int v = tid + i * kThreads;
-      const int r = v / 8, c = v % 8;
+      const int r = v / CPR, c = v % CPR;
       const int row = key0 + r < seq ? key0 + r : seq - 1;
       rk[i] = *reinterpret_cast<const half8 *>(kBase + int64_t(row) * tokStride + c * 8);
       rv[i] = *reinterpret_cast<const half8 *>(vBase + int64_t(row) * tokStride + c * 8);
@@ -171,16 +184,17 @@ __attribute__((amdgpu_waves_per_eu(2, KS == 1 ? 4 : 2))) void bertAttentionKerne
       for (int e = 0; e < 4; e++)
         z[e] = _Float16(0);
 #pragma unroll
-      for (int c = 0; c < 8; c++)
+      for (int c = 0; c < CPR; c++)
         *reinterpret_cast<half4 *>(oBase + int64_t(q) * outStride + c * 8 +
                                    hb * 4) = z;
     }
     return;
   }
 
-  float16v accO[2]; // O^T: two 32-wide d blocks
+  constexpr int DB = D / 32;
+  float16v accO[DB]; // O^T: 32-wide d blocks
 #pragma unroll
-  for (int d = 0; d < 2; d++)
+  for (int d = 0; d < DB; d++)
 #pragma unroll
     for (int e = 0; e < 16; e++)
       accO[d][e] = 0.f;
@@ -189,20 +203,21 @@ __attribute__((amdgpu_waves_per_eu(2, KS == 1 ? 4 : 2))) void bertAttentionKerne
   const float scaleLog2e = scale * 1.44269504088896340736f;
 
   // Per-lane constants of the fragment addresses.
-  const int swzLane = (l32 >> 1) & 7;          // K: (row >> 1) & 7 for row = 32*x + l32
+  const int swzLane = swzK<D>(l32, 0);         // K: the row term for row = 32*x + l32
   const int trRow = (lane % 16) / 4;           // V: source row inside a run of 4 keys
   const int trCol = ((lane % 32) / 16) * 16 + (lane % 4) * 4;
-  const int vSwz = (trRow >> 1) & 1;           // key bases are multiples of 4
+  const int vSwz = swzV<D>(trRow, 0);          // key bases are multiples of 4
 
   // Staging without prefetch: thread t copies 16-byte vector t % 8 of rows
   // t / 8 + i * kThreads / 8.  Both swizzles depend on row bits that the
   // per-vector row step (a multiple of 16) leaves alone, so the LDS
   // destinations are one base plus immediates.
   const uint32_t rowBytes = uint32_t(tokStride) * 2u;
-  const uint32_t stageOff = uint32_t(tid / 8) * rowBytes + uint32_t(tid % 8) * 16u;
-  const int stageK = (tid / 8) * 128 + swzK(tid / 8, tid % 8) * 16;
-  const int stageV =
-      (tid / 8) * 128 + swzV(tid / 8, (tid % 8) / 4) * 64 + ((tid % 8) % 4) * 16;
+  const uint32_t stageOff = uint32_t(tid / CPR) * rowBytes + uint32_t(tid % CPR) * 16u;
+  const int stageK = (tid / CPR) * kRowB + swzK<D>(tid / CPR, tid % CPR) * 16;
+  const int stageV = (tid / CPR) * kRowB + swzV<D>(tid / CPR, (tid % CPR) / 4) * 64 +
+                     ((tid % CPR) % 4) * 16;
+  static_assert((kThreads / CPR) % 16 == 0, "row step per vector must leave the swizzles alone");
   const auto rsrcK = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<_Float16 *>(kBase), 0, int32_t(uint32_t(len) * rowBytes),
       0x00020000);
@@ -230,7 +245,7 @@ __attribute__((amdgpu_waves_per_eu(2, KS == 1 ? 4 : 2))) void bertAttentionKerne
 #pragma unroll
       for (int i = 0; i < VPT; i++) {
         const int v = tid + i * kThreads;
-        const int r = v / 8, c = v % 8;
+        const int r = v / CPR, c = v % CPR;
         if (r < live) {
           half8 kv = rk[i], vv = rv[i];
           if (key0 + r >= len) {
@@ -238,8 +253,8 @@ __attribute__((amdgpu_waves_per_eu(2, KS == 1 ? 4 : 2))) void bertAttentionKerne
             for (int e = 0; e < 8; e++)
               kv[e] = vv[e] = _Float16(0);
           }
-          *reinterpret_cast<half8 *>(sK + r * 128 + swzK(r, c) * 16) = kv;
-          *reinterpret_cast<half8 *>(sV + r * 128 + swzV(r, c / 4) * 64 + (c % 4) * 16) = vv;
+          *reinterpret_cast<half8 *>(sK + r * kRowB + swzK<D>(r, c) * 16) = kv;
+          *reinterpret_cast<half8 *>(sV + r * kRowB + swzV<D>(r, c / 4) * 64 + (c % 4) * 16) = vv;
         }
       }
     } else {
@@ -250,7 +265,7 @@ __attribute__((amdgpu_waves_per_eu(2, KS == 1 ? 4 : 2))) void bertAttentionKerne
       const uint32_t chunkOff = stageOff + uint32_t(key0) * rowBytes;
 #pragma unroll
       for (int i = 0; i < VPT; i++) {
-        const uint32_t off = chunkOff + uint32_t(i * (kThreads / 8)) * rowBytes;
+        const uint32_t off = chunkOff + uint32_t(i * (kThreads / CPR)) * rowBytes;
         kv[i] = __builtin_bit_cast(
             half8, __builtin_amdgcn_raw_buffer_load_b128(rsrcK, off, 0, 0));
         vv[i] = __builtin_bit_cast(
@@ -258,8 +273,8 @@ __attribute__((amdgpu_waves_per_eu(2, KS == 1 ? 4 : 2))) void bertAttentionKerne
       }
 #pragma unroll
       for (int i = 0; i < VPT; i++) {
-        *reinterpret_cast<half8 *>(sK + stageK + i * (kThreads / 8) * 128) = kv[i];
-        *reinterpret_cast<half8 *>(sV + stageV + i * (kThreads / 8) * 128) = vv[i];
+        *reinterpret_cast<half8 *>(sK + stageK + i * (kThreads / CPR) * kRowB) = kv[i];
+        *reinterpret_cast<half8 *>(sV + stageV + i * (kThreads / CPR) * kRowB) = vv[i];
       }
     }
     if (kPrefetch && ch + 1 < numChunks)
@@ -276,7 +291,7 @@ __attribute__((amdgpu_waves_per_eu(2, KS == 1 ? 4 : 2))) void bertAttentionKerne
 #pragma unroll
         for (int kk = 0; kk < kHeadDim / 16; kk++)
           fk[sb][kk] = *reinterpret_cast<const half8 *>(
-              sK + (blk + sb * 32 + l32) * 128 + ((kk * 2 + hb) ^ swzLane) * 16);
+              sK + (blk + sb * 32 + l32) * kRowB + ((kk * 2 + hb) ^ swzLane) * 16);
       __builtin_amdgcn_sched_barrier(0);
       float16v accS[2];
 #pragma unroll
@@ -329,7 +344,7 @@ __attribute__((amdgpu_waves_per_eu(2, KS == 1 ? 4 : 2))) void bertAttentionKerne
         rowSum *= corr;
         rowMax = newMax;
 #pragma unroll
-        for (int d = 0; d < 2; d++)
+        for (int d = 0; d < DB; d++)
 #pragma unroll
           for (int e = 0; e < 16; e++)
             accO[d][e] *= corr;
@@ -360,7 +375,7 @@ __attribute__((amdgpu_waves_per_eu(2, KS == 1 ? 4 : 2))) void bertAttentionKerne
           for (int e = 0; e < 8; e++)
             fp[e] = _Float16(accS[sb][8 * t + e]);
 #pragma unroll
-          for (int d = 0; d < 2; d++) {
+          for (int d = 0; d < DB; d++) {
             // A operand: V[key(hb, e)][d*32 + l32]: two runs of 4 consecutive
             // keys, each transposed out of 4 V rows x 16 columns by one read.
             short4v run[2];
@@ -369,7 +384,7 @@ __attribute__((amdgpu_waves_per_eu(2, KS == 1 ? 4 : 2))) void bertAttentionKerne
               const int keyLocal = blk + sb * 32 + 8 * (2 * t + g) + 4 * hb + trRow;
               run[g] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
                   (__attribute__((address_space(3))) short4v *)(
-                      sV + keyLocal * 128 + (d ^ vSwz) * 64 + trCol * 2));
+                      sV + keyLocal * kRowB + (d ^ vSwz) * 64 + trCol * 2));
             }
             short8v both;
 #pragma unroll
@@ -393,28 +408,29 @@ __attribute__((amdgpu_waves_per_eu(2, KS == 1 ? 4 : 2))) void bertAttentionKerne
   // sums.  A share that saw no valid key has m1 = -inf and weight 0; share 0
   // always owns the first block, which has one.
   if constexpr (KS == 2) {
-    static_assert(QG * 34 * kWave * 4 <= 2 * kTileBytes, "exchange fits the K/V tiles");
-    float *xch = reinterpret_cast<float *>(smem) + qg * (34 * kWave) + lane;
+    constexpr int XV = DB * 16; // accumulator values per lane
+    static_assert(QG * (XV + 2) * kWave * 4 <= 2 * kTileBytes, "exchange fits the K/V tiles");
+    float *xch = reinterpret_cast<float *>(smem) + qg * ((XV + 2) * kWave) + lane;
     __syncthreads(); // every wavefront is done with K and V
     if (kh == 1) {
 #pragma unroll
-      for (int d = 0; d < 2; d++)
+      for (int d = 0; d < DB; d++)
 #pragma unroll
         for (int e = 0; e < 16; e++)
           xch[(d * 16 + e) * kWave] = accO[d][e];
-      xch[32 * kWave] = rowMax;
-      xch[33 * kWave] = rowSum;
+      xch[XV * kWave] = rowMax;
+      xch[(XV + 1) * kWave] = rowSum;
     }
     __syncthreads();
     if (kh == 1)
       return;
-    const float m1 = xch[32 * kWave], l1 = xch[33 * kWave];
+    const float m1 = xch[XV * kWave], l1 = xch[(XV + 1) * kWave];
     const float m = fmaxf(rowMax, m1);
     const float c0 = __builtin_amdgcn_exp2f((rowMax - m) * scaleLog2e);
     const float c1 = __builtin_amdgcn_exp2f((m1 - m) * scaleLog2e);
     rowSum = rowSum * c0 + l1 * c1;
 #pragma unroll
-    for (int d = 0; d < 2; d++)
+    for (int d = 0; d < DB; d++)
 #pragma unroll
       for (int e = 0; e < 16; e++)
         accO[d][e] = accO[d][e] * c0 + xch[(d * 16 + e) * kWave] * c1;
@@ -427,7 +443,7 @@ __attribute__((amdgpu_waves_per_eu(2, KS == 1 ? 4 : 2))) void bertAttentionKerne
     const bool valid = q < len;
     const float inv = valid ? 1.0f / rowSum : 0.f;
 #pragma unroll
-    for (int d = 0; d < 2; d++)
+    for (int d = 0; d < DB; d++)
 #pragma unroll
       for (int g = 0; g < 4; g++) {
         half4 o;
@@ -446,8 +462,10 @@ Status launchBertAttentionF16(const _Float16 *qkv, const int32_t *cuSeqlens,
                               _Float16 *out, int64_t bs, int64_t seq,
                               int64_t heads, int64_t headDim, float scale,
                               hipStream_t s) {
-  HOM_CHECK_RET(headDim == kHeadDim, Status::kInvalidArgument,
-                "attention: head size %lld not supported (only 64)",
+  // (the reference's contract is head size % 64 == 0, README.md:11; the
+  // sizes with kernels here are 64 and 128)
+  HOM_CHECK_RET(headDim == 64 || headDim == 128, Status::kInvalidArgument,
+                "attention: head size %lld not supported (64 or 128)",
                 (long long)headDim);
   // The softmax tracks the maximum of the unscaled scores, which is the
   // maximum of the scaled ones only for a positive scale (BERT: 1/sqrt(64)).
@@ -456,7 +474,7 @@ Status launchBertAttentionF16(const _Float16 *qkv, const int32_t *cuSeqlens,
   HOM_CHECK_RET(bs < 65536 && heads < 65536 && seq < (int64_t(1) << 24),
                 Status::kInvalidArgument, "attention: shape out of range");
   // K/V staging addresses a batch entry with 32-bit byte offsets
-  HOM_CHECK_RET(seq * 3 * heads * kHeadDim * 2 < (int64_t(1) << 31),
+  HOM_CHECK_RET(seq * 3 * heads * headDim * 2 < (int64_t(1) << 31),
                 Status::kInvalidArgument,
                 "attention: one batch entry of QKV must be smaller than 2 GiB");
   HOM_CHECK_RET((reinterpret_cast<uintptr_t>(qkv) & 15) == 0 &&
@@ -477,15 +495,24 @@ Status launchBertAttentionF16(const _Float16 *qkv, const int32_t *cuSeqlens,
                 Status::kInvalidArgument, "attention: too many workgroups");
   if (wide) {
     const int nq = int((seq + 127) / 128);
-    bertAttentionKernel<4, 1><<<dim3((unsigned)(nq * pairs)), dim3(256), 0, s>>>(
-        qkv, cuSeqlens, out, int(seq), int(heads), nq, int(pairs), scale);
+    const dim3 grid((unsigned)(nq * pairs));
+    if (headDim == 64)
+      bertAttentionKernel<4, 1, 64><<<grid, dim3(256), 0, s>>>(
+          qkv, cuSeqlens, out, int(seq), int(heads), nq, int(pairs), scale);
+    else
+      bertAttentionKernel<4, 1, 128><<<grid, dim3(256), 0, s>>>(
+          qkv, cuSeqlens, out, int(seq), int(heads), nq, int(pairs), scale);
   } else {
     const int nq = int((seq + 63) / 64);
     HOM_CHECK_RET(heads < 65536 && bs < 65536, Status::kInvalidArgument,
                   "attention: heads and batch size must be below 65536");
-    bertAttentionKernel<4, 2>
-        <<<dim3((unsigned)nq, (unsigned)heads, (unsigned)bs), dim3(256), 0, s>>>(
-            qkv, cuSeqlens, out, int(seq), int(heads), nq, int(pairs), scale);
+    const dim3 grid((unsigned)nq, (unsigned)heads, (unsigned)bs);
+    if (headDim == 64)
+      bertAttentionKernel<4, 2, 64><<<grid, dim3(256), 0, s>>>(
+          qkv, cuSeqlens, out, int(seq), int(heads), nq, int(pairs), scale);
+    else
+      bertAttentionKernel<4, 2, 128><<<grid, dim3(256), 0, s>>>(
+          qkv, cuSeqlens, out, int(seq), int(heads), nq, int(pairs), scale);
   }
   HOM_HIP_RET(hipGetLastError(), Status::kInternal);
   return Status::kSuccess;
