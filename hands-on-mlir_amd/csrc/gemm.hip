@@ -4,6 +4,7 @@
 // python/gemm_generator.py:237-278).  The kernels themselves are templates in
 // gemm_dma.h / gemm_pipe.h / gemm_staged.h, instantiated in gemm_inst_*.hip.
 #include "gemm_dma.h"
+#include "gemm_fine.h"
 #include "gemm_pipe.h"
 #include "gemm_staged.h"
 
@@ -35,6 +36,8 @@ namespace gemmk {
 #define HOM_PIPE_TILE_B HOM_PIPE_TILE_A
 #define HOM_PIPE_TILE_C HOM_PIPE_TILE_A
 #define HOM_PIPE_TILE_D HOM_PIPE_TILE_A
+#define HOM_FINE_TILE(BM, BN, WM, WN, DIST)                                    \
+  HOM_EXTERN_EPILOGUES(launchFine, BM, BN, WM, WN, DIST)
 #define HOM_STAGED_TILE(BM, BN, BK, WM, WN, VEC)                               \
   HOM_EXTERN_STAGED(BM, BN, BK, WM, WN, 0, VEC)                                \
   HOM_EXTERN_STAGED(BM, BN, BK, WM, WN, 1, VEC)                                \
@@ -45,6 +48,7 @@ namespace gemmk {
 #undef HOM_PIPE_TILE_B
 #undef HOM_PIPE_TILE_C
 #undef HOM_PIPE_TILE_D
+#undef HOM_FINE_TILE
 #undef HOM_STAGED_TILE
 } // namespace gemmk
 
@@ -108,6 +112,21 @@ struct KernelEntry {
 #define HOM_PIPE_TILE_B HOM_PIPE_TILE_A
 #define HOM_PIPE_TILE_C HOM_PIPE_TILE_A
 #define HOM_PIPE_TILE_D HOM_PIPE_TILE_A
+
+// The 16x16x32-MFMA family ("s16x16x32" in the name); N and the leading
+// dimensions of B, C, D must be multiples of 8.
+#define HOM_FINE_ENTRY(BM, BN, WM, WN, DIST, EPI_ENUM, EPI_STR, ACT)           \
+  {                                                                            \
+    {"hom_gfx950_mfma_f16_s16x16x32gemm_f16_" #BM "x" #BN "_64x2r" #DIST       \
+     "_w" #WM "x" #WN "_nn_align8_" EPI_STR,                                   \
+     BM, BN, 64, WM, WN, 8, 8, ACT, EPI_ENUM},                                 \
+        launchFine<BM, BN, WM, WN, DIST, int(EPI_ENUM), false>,                \
+        launchFine<BM, BN, WM, WN, DIST, int(EPI_ENUM), true>                  \
+  }
+#define HOM_FINE_TILE(BM, BN, WM, WN, DIST)                                    \
+  HOM_FINE_ENTRY(BM, BN, WM, WN, DIST, Epilogue::kLinear, "linear", 0),        \
+      HOM_FINE_ENTRY(BM, BN, WM, WN, DIST, Epilogue::kGeluErf, "gelu", 1),     \
+      HOM_FINE_ENTRY(BM, BN, WM, WN, DIST, Epilogue::kGeluTanh, "gelutanh", 1),
 
 // Manifest order is part of the ABI: compiled modules carry indices into it.
 // New entries go at the end of gemm_manifest.inc.

@@ -17,4 +17,5 @@
 #define HOM_PIPE_TILE_B(...)
 #define HOM_PIPE_TILE_C(...)
 #define HOM_PIPE_TILE_D(...)
+#define HOM_FINE_TILE(...)
 #define HOM_STAGED_TILE(...)

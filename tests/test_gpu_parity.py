@@ -186,6 +186,52 @@ def test_gemm_every_manifest_kernel(gpu, rt, oracle):
                 assert_close(got[0], want, **GEMM_TOL, what=f"{name} {M_}x{N_}x{K_} splitK={sk}")
 
 
+FINE_TILES = ("128x96_64x2r2_w4x2", "64x48_64x2r2_w4x1", "64x48_64x2r4_w4x1", "64x144_64x2r2_w4x1")
+
+
+def test_gemm_fine_family(gpu, rt, oracle, monkeypatch):
+    """The 16x16x32-MFMA kernels (tile sides in steps of 16): every epilogue source form (none, bias row,
+    in-place residual, a [M', N] source shared by the batch entries = the general epilogue), GELU, split-K,
+    ragged M / N / K, more tiles than CUs, and the [N, K] layout of B through nvteGemmF16."""
+    g = np.random.default_rng(41)
+    M = rt.MemRef.from_tensor
+    for tile in FINE_TILES:
+        for (M_, N_, K_) in [(256, 288, 128), (200, 264, 136), (72, 40, 392), (1100, 2000, 72)]:
+            A = g.standard_normal((1, M_, K_)).astype(np.float16)
+            B = (g.standard_normal((1, K_, N_)) * 0.1).astype(np.float16)
+            bias = g.standard_normal((1, 1, N_)).astype(np.float16)
+            R = g.standard_normal((1, M_, N_)).astype(np.float16)
+            want_bias = oracle.gemm(A[0], B[0], bias[0], beta=1.0, act="gelu_erf")
+            want_res = oracle.gemm(A[0], B[0], R[0], beta=0.5, alpha=2.0)
+            for sk in (1, 2):
+                got = run_gemm(gpu, rt, A, B, bias, np.zeros((1, M_, N_), np.float16), knum(rt, tile, "gelu"), sk,
+                               beta=1.0)
+                assert_close(got[0], want_bias, **GEMM_TOL, what=f"{tile} splitK={sk} {M_}x{N_}x{K_} bias+gelu")
+                got = run_gemm(gpu, rt, A, B, None, R, knum(rt, tile), sk, alpha=2.0, beta=0.5, in_place=True)
+                assert_close(got[0], want_res, **GEMM_TOL, what=f"{tile} splitK={sk} {M_}x{N_}x{K_} residual")
+        # batch of 3 with one [M', N] source shared by the entries (the source-row period form)
+        b, Mp, N_, K_ = 3, 40, 96, 64
+        A = g.standard_normal((b, Mp, K_)).astype(np.float16)
+        B = (g.standard_normal((1, K_, N_)) * 0.1).astype(np.float16)
+        C = g.standard_normal((1, Mp, N_)).astype(np.float16)
+        want = oracle.gemm(A.reshape(-1, K_), B[0], np.tile(C[0], (b, 1)), beta=1.0, act="gelu_tanh")
+        got = run_gemm(gpu, rt, A, B, C, np.zeros((b, Mp, N_), np.float16), knum(rt, tile, "gelutanh"), 1, beta=1.0)
+        assert_close(got.reshape(-1, N_), want, **GEMM_TOL, what=f"{tile} shared source")
+        # B as [N, K]
+        name = [n for _, n, _, _ in rt.manifest() if f"_{tile}_" in n and n.endswith("_linear")][0]
+        for (b, Mp, K_, N_, beta, sk) in [(2, 100, 136, 264, 1.0, 1), (1, 256, 128, 288, 0.0, 2)]:
+            monkeypatch.setenv("HOM_NVTE_GEMM_KERNEL", f"{name},{sk}")
+            A = g.standard_normal((b, Mp, K_)).astype(np.float16)
+            Bt = (g.standard_normal((1, N_, K_)) * 0.05).astype(np.float16)
+            X = g.standard_normal((b, Mp, N_)).astype(np.float16)
+            want = oracle.gemm(A.reshape(-1, K_), Bt[0], X.reshape(-1, N_), beta=beta, b_is_nk=True)
+            ta, tb, td = dev(A), dev(Bt), dev(X)
+            gpu.nvteGemmF16(*M(ta).args(), False, *M(tb).args(), True, *M(td).args(), *M(td).args(),
+                            0, 1.0, beta, 0, 0)
+            assert_close(host(td).reshape(-1, N_), want, **GEMM_TOL, what=f"{tile} [N,K] {Mp}x{N_}x{K_} splitK={sk}")
+        monkeypatch.delenv("HOM_NVTE_GEMM_KERNEL")
+
+
 def test_gemm_more_tiles_than_resident_workgroups(gpu, rt, oracle):
     """Ragged problem whose tile count exceeds what the chip holds at once, so the
     persistent kernels walk several tiles per workgroup (with and without split-K)."""
