@@ -25,6 +25,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <chrono>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -510,7 +511,8 @@ DRV_EXPORT int homBertSetGemmChoice(HomBertEncoder *e, int role,
 
 // ---- single-operator timing through the boundary -------------------------
 // Each helper enqueues `iters` back-to-back calls of one entry point between
-// two events on a private stream and returns mean milliseconds per call.
+// two events on a private stream, behind a warm-up (Timer::warm), and returns
+// mean milliseconds per call.
 
 namespace {
 struct Timer {
@@ -535,12 +537,29 @@ struct Timer {
       (void)hipStreamDestroy(s);
     }
   }
+  // Untimed calls before the timed ones: at least `warmup`, and as many as it
+  // takes to keep the GPU busy for kMinWarmMs.  After an idle period (the
+  // uploads that precede a timing loop are one) the first tens of
+  // milliseconds of launches run slower than the steady state: 10.1 us per
+  // launch against 8.7 us for the 1024 x 3072 x 768 GEMM.
+  static constexpr double kMinWarmMs = 150.0;
+  template <typename F> bool warm(F &&fn, int warmup) {
+    const auto t0 = std::chrono::steady_clock::now();
+    const int batch = warmup > 10 ? warmup : 10;
+    for (;;) {
+      for (int i = 0; i < batch; i++)
+        fn();
+      if (!hipOk(hipStreamSynchronize(s), "sync"))
+        return false;
+      const double ms = std::chrono::duration<double, std::milli>(
+                            std::chrono::steady_clock::now() - t0)
+                            .count();
+      if (ms >= kMinWarmMs)
+        return true;
+    }
+  }
   template <typename F> double run(F &&fn, int iters, int warmup) {
-    if (!ok)
-      return -1.0;
-    for (int i = 0; i < warmup; i++)
-      fn();
-    if (!hipOk(hipStreamSynchronize(s), "sync"))
+    if (!ok || !warm(fn, warmup))
       return -1.0;
     (void)hipEventRecord(a, s);
     for (int i = 0; i < iters; i++)
@@ -551,6 +570,45 @@ struct Timer {
     float ms = 0.f;
     (void)hipEventElapsedTime(&ms, a, b);
     return double(ms) / double(iters > 0 ? iters : 1);
+  }
+  // The same calls as kernel nodes of a HIP graph: `perGraph` calls are
+  // captured once and the graph is replayed `replays` times between the
+  // events.  Inside a graph a dependent launch costs less than on a stream,
+  // and a graph is how the encoder's call list runs.
+  template <typename F>
+  double runGraph(F &&fn, int perGraph, int replays, int warmup) {
+    if (!ok)
+      return -1.0;
+    fn(); // sizes whatever scratch the call needs before the capture
+    if (!hipOk(hipStreamSynchronize(s), "sync"))
+      return -1.0;
+    hipGraph_t g = nullptr;
+    hipGraphExec_t ge = nullptr;
+    if (!hipOk(hipStreamBeginCapture(s, hipStreamCaptureModeRelaxed), "capture"))
+      return -1.0;
+    for (int i = 0; i < perGraph; i++)
+      fn();
+    double out = -1.0;
+    if (hipOk(hipStreamEndCapture(s, &g), "end capture") &&
+        hipOk(hipGraphInstantiate(&ge, g, nullptr, nullptr, 0), "instantiate")) {
+      if (warm([&] { (void)hipGraphLaunch(ge, s); }, warmup)) {
+        (void)hipEventRecord(a, s);
+        for (int i = 0; i < replays; i++)
+          (void)hipGraphLaunch(ge, s);
+        (void)hipEventRecord(b, s);
+        if (hipOk(hipEventSynchronize(b), "event sync")) {
+          float ms = 0.f;
+          (void)hipEventElapsedTime(&ms, a, b);
+          out = double(ms) / double(replays > 0 ? replays : 1) /
+                double(perGraph > 0 ? perGraph : 1);
+        }
+      }
+    }
+    if (ge)
+      (void)hipGraphExecDestroy(ge);
+    if (g)
+      (void)hipGraphDestroy(g);
+    return out;
   }
 };
 
@@ -574,10 +632,11 @@ void fillRandomF16(void *dev, int64_t numel, float scale, uint32_t seed) {
 } // namespace
 
 // D = act(A.B + bias) with bias broadcast as a [1,1,N] C (useBias) or beta = 0.
-// gemmNum is 1-based (0 = library picks); returns ms per call.
-DRV_EXPORT double homTimeGemm(int64_t M, int64_t N, int64_t K, int64_t act,
-                              int useBias, int32_t gemmNum, int32_t splitK,
-                              int iters, int warmup) {
+// gemmNum is 1-based (0 = library picks); returns ms per call.  inGraph != 0:
+// 100 calls per captured graph, iters / 100 replays.
+static double timeGemm(int64_t M, int64_t N, int64_t K, int64_t act,
+                       int useBias, int32_t gemmNum, int32_t splitK, int iters,
+                       int warmup, int inGraph) {
   Tensor a, b, c, d;
   a.m = alloc3DMemRefNVGPUF16(1, int32_t(M), int32_t(K));
   b.m = alloc3DMemRefNVGPUF16(1, int32_t(K), int32_t(N));
@@ -589,20 +648,32 @@ DRV_EXPORT double homTimeGemm(int64_t M, int64_t N, int64_t K, int64_t act,
   double ms;
   {
     Timer t;
-    ms = t.run(
-        [&] {
-          cutlassGemmF16(3, a.m.descriptor, false, 3, b.m.descriptor, false, 3,
-                         useBias ? c.m.descriptor : d.m.descriptor, 3,
-                         d.m.descriptor, act, 1.0f, useBias ? 1.0f : 0.0f,
-                         gemmNum, splitK);
-        },
-        iters, warmup);
+    auto call = [&] {
+      cutlassGemmF16(3, a.m.descriptor, false, 3, b.m.descriptor, false, 3,
+                     useBias ? c.m.descriptor : d.m.descriptor, 3,
+                     d.m.descriptor, act, 1.0f, useBias ? 1.0f : 0.0f, gemmNum,
+                     splitK);
+    };
+    ms = inGraph ? t.runGraph(call, 100, (iters + 99) / 100, (warmup + 99) / 100)
+                 : t.run(call, iters, warmup);
   }
   a.release();
   b.release();
   c.release();
   d.release();
   return ms;
+}
+
+DRV_EXPORT double homTimeGemm(int64_t M, int64_t N, int64_t K, int64_t act,
+                              int useBias, int32_t gemmNum, int32_t splitK,
+                              int iters, int warmup) {
+  return timeGemm(M, N, K, act, useBias, gemmNum, splitK, iters, warmup, 0);
+}
+
+DRV_EXPORT double homTimeGemmInGraph(int64_t M, int64_t N, int64_t K,
+                                     int64_t act, int useBias, int32_t gemmNum,
+                                     int32_t splitK, int iters, int warmup) {
+  return timeGemm(M, N, K, act, useBias, gemmNum, splitK, iters, warmup, 1);
 }
 
 // Same through nvteGemmF16 (B given as [1, N, K]); the library picks the kernel.
