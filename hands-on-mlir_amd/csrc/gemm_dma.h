@@ -44,10 +44,8 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmDmaKernel(GemmParams p) {
   const int waveM = wave / WN, waveN = wave % WN;
   const int l32 = lane % 32, kb = lane / 32;
 
-  const int nTiles = p.tilesM * p.tilesN;
-  const int tile = tileForBlock(nTiles, blockIdx.x);
   int tileM, tileN;
-  tileCoords(tile, p.tilesM, p.tilesN, &tileM, &tileN);
+  const int tile = tileCoordsFast(p, int(blockIdx.x), &tileM, &tileN);
   const int m0 = tileM * BM, n0 = tileN * BN;
   const int slice = blockIdx.y, numSlices = gridDim.y;
   const int kTiles = (p.K + BK - 1) / BK;
@@ -76,6 +74,14 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmDmaKernel(GemmParams p) {
   // rejects such problems for these kernels.
 
   // ---- per-lane source offsets (bytes), constant over the K walk ----
+  // A slab's loads are one constant 32-bit offset per lane plus a scalar
+  // offset per slab: the main loop computes no addresses and tests no ranges.
+  // Rows past M (or N, for B as [N, K]) lie beyond the descriptor and read as
+  // zero; columns of a row-major B past N get an offset beyond every
+  // descriptor; rows of a row-major B past K lie beyond its descriptor.  Only
+  // the partial last slab of a ragged K needs a test per lane (issueChecked).
+  const int kEnd = ktEnd * BK < p.K ? ktEnd * BK : p.K;
+  const int ktPartial = kEnd % BK != 0 ? ktEnd - 1 : -1;
   uint32_t aOff[A_PER_W];
   int aCol[A_PER_W];
 #pragma unroll
@@ -84,10 +90,10 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmDmaKernel(GemmParams p) {
     const int r = instr * 8 + lane / 8;
     const int c = swzK(r, lane % 8); // logical chunk stored at this position
     aCol[i] = c * 8;
-    aOff[i] = (m0 + r < p.M) ? uint32_t((int64_t(r) * p.lda + c * 8) * 2) : kOob;
+    aOff[i] = (uint32_t(r) * uint32_t(p.lda) + uint32_t(c * 8)) * 2u;
   }
   uint32_t bOff[B_PER_W];
-  int bK[B_PER_W]; // NK: column offset in k; KN: row (k) inside the slab
+  int bK[B_PER_W]; // NK: column offset in k (KN: unused)
 #pragma unroll
   for (int i = 0; i < B_PER_W; i++) {
     const int instr = wave * B_PER_W + i;
@@ -95,15 +101,17 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmDmaKernel(GemmParams p) {
       const int r = instr * 8 + lane / 8;
       const int c = swzK(r, lane % 8);
       bK[i] = c * 8;
-      bOff[i] = (n0 + r < p.N) ? uint32_t((int64_t(r) * p.ldb + c * 8) * 2) : kOob;
+      bOff[i] = (uint32_t(r) * uint32_t(p.ldb) + uint32_t(c * 8)) * 2u;
     } else {
       constexpr int CHUNKS = B_ROW_BYTES / 16;
       const int k = instr * B_ROWS_PER_INSTR + lane / CHUNKS;
       const int pc = lane % CHUNKS; // physical chunk
       const int g = swzN<BN>(k, pc / 4);
       const int n = (g * 4 + pc % 4) * 8;
-      bK[i] = k;
-      bOff[i] = (n0 + n < p.N) ? uint32_t((int64_t(k) * p.ldb + n0 + n) * 2) : kOob;
+      bK[i] = 0;
+      bOff[i] = (n0 + n < p.N)
+                    ? (uint32_t(k) * uint32_t(p.ldb) + uint32_t(n0 + n)) * 2u
+                    : kOob;
     }
   }
 
@@ -111,28 +119,31 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmDmaKernel(GemmParams p) {
     unsigned char *sA = smem + stage * STAGE_BYTES;
     unsigned char *sB = sA + A_BYTES;
     const int k0 = kt * BK;
-    const bool live = kt < ktEnd;
+    const uint32_t sOffA = uint32_t(k0) * 2u;
+    const uint32_t sOffB = B_NK ? sOffA : uint32_t(k0) * uint32_t(p.ldb) * 2u;
+    if (kt != ktPartial) {
 #pragma unroll
-    for (int i = 0; i < A_PER_W; i++) {
-      const uint32_t off = (live && k0 + aCol[i] < p.K && aOff[i] != kOob)
-                               ? aOff[i] + uint32_t(k0) * 2u
-                               : kOob;
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(
-          rsrcA, HOM_LDS_PTR(sA + (wave * A_PER_W + i) * 1024), 16, off, 0, 0, 0);
-    }
+      for (int i = 0; i < A_PER_W; i++)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(
+            rsrcA, HOM_LDS_PTR(sA + (wave * A_PER_W + i) * 1024), 16, aOff[i],
+            sOffA, 0, 0);
 #pragma unroll
-    for (int i = 0; i < B_PER_W; i++) {
-      uint32_t off;
-      if (B_NK)
-        off = (live && k0 + bK[i] < p.K && bOff[i] != kOob)
-                  ? bOff[i] + uint32_t(k0) * 2u
-                  : kOob;
-      else
-        off = (live && k0 + bK[i] < p.K && bOff[i] != kOob)
-                  ? bOff[i] + uint32_t(int64_t(k0) * p.ldb * 2)
-                  : kOob;
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(
-          rsrcB, HOM_LDS_PTR(sB + (wave * B_PER_W + i) * 1024), 16, off, 0, 0, 0);
+      for (int i = 0; i < B_PER_W; i++)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(
+            rsrcB, HOM_LDS_PTR(sB + (wave * B_PER_W + i) * 1024), 16, bOff[i],
+            sOffB, 0, 0);
+    } else {
+      // the partial slab: vectors at or past the end of K read as zero
+#pragma unroll
+      for (int i = 0; i < A_PER_W; i++)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(
+            rsrcA, HOM_LDS_PTR(sA + (wave * A_PER_W + i) * 1024), 16,
+            k0 + aCol[i] < kEnd ? aOff[i] : kOob, sOffA, 0, 0);
+#pragma unroll
+      for (int i = 0; i < B_PER_W; i++)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(
+            rsrcB, HOM_LDS_PTR(sB + (wave * B_PER_W + i) * 1024), 16,
+            (!B_NK || k0 + bK[i] < kEnd) ? bOff[i] : kOob, sOffB, 0, 0);
     }
   };
 
@@ -205,26 +216,41 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmDmaKernel(GemmParams p) {
   };
 
   // ---- main loop: NS-deep ring of slabs, one barrier per slab ----
-  // Every wavefront issues exactly LOADS_PER_TILE DMA loads per slab (slabs past
-  // the end are all out of range and write zeros), so "slab i+1 has landed" is
-  // vmcnt <= (NS-2) * LOADS_PER_TILE once slabs up to i+NS-1 have been issued.
-  // Inside a slab the fragments of k step kk+1 are fetched from LDS before the
-  // MFMAs of step kk are issued (two register sets), and the barrier that frees
-  // the slab's LDS buffer sits between the last fragment fetch and the last
-  // MFMA group, so the matrix core keeps running while the wavefronts
+  // A wavefront issues LOADS_PER_TILE DMA loads per slab, in slab order, so
+  // "slab j has landed for this wavefront" is vmcnt <= LOADS_PER_TILE x (slabs
+  // issued after j); the barrier behind that wait makes it true for the whole
+  // workgroup.  Slabs that do not exist are not issued, and the wait counts
+  // what was.  Inside a slab the fragments of k step kk+1 are fetched from LDS
+  // before the MFMAs of step kk are issued (two register sets), and the barrier
+  // that frees the slab's LDS buffer sits between the last fragment fetch and
+  // the last MFMA group, so the matrix core keeps running while the wavefronts
   // synchronise, refill the ring and fetch the next slab's first fragments.
-  // The waits and the barrier are one opaque asm statement with a memory
-  // clobber: the compiler may not move LDS reads or DMA issues across it.
-  constexpr int kInFlight = (NS - 2) * LOADS_PER_TILE;
+  // The waits and the barrier are opaque asm statements with a memory clobber:
+  // the compiler may not move LDS reads or DMA issues across them.
   constexpr int KSTEPS = BK / 16;
+  auto waitOutstanding = [&](int slabs) { // wave-uniform, 0 .. NS-2
+    staticFor<NS - 1>([&](auto vC) {
+      constexpr int v = decltype(vC)::value;
+      if (slabs == v)
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(v * LOADS_PER_TILE) : "memory");
+    });
+  };
   half8 fa[2][MI], fb[2][NI];
-#pragma unroll
-  for (int s = 0; s < NS - 1; s++)
-    issue(ktBegin + s, s);
   const int nk = ktEnd - ktBegin;
   if (nk > 0) {
-    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(kInFlight) : "memory");
-    issue(ktBegin + NS - 1, NS - 1);
+    int issued = 0;
+#pragma unroll
+    for (int s0 = 0; s0 < NS - 1; s0++)
+      if (s0 < nk) {
+        issue(ktBegin + s0, s0);
+        issued = s0 + 1;
+      }
+    waitOutstanding(issued - 1); // slab 0
+    asm volatile("s_barrier" ::: "memory");
+    if (issued < nk) {
+      issue(ktBegin + issued, issued % NS);
+      issued++;
+    }
     loadFrags(0, 0, fa[0], fb[0]);
     for (int i = 0; i < nk; i++) {
       const int cur = i % NS;
@@ -236,10 +262,13 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmDmaKernel(GemmParams p) {
       if (i + 1 < nk) {
         // all of this wavefront's reads of slab i are in registers; slab i+1
         // has landed for this wavefront; then wait for the other wavefronts
-        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(
-                         kInFlight)
-                     : "memory");
-        issue(ktBegin + i + NS, cur);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        waitOutstanding(issued - i - 2);
+        asm volatile("s_barrier" ::: "memory");
+        if (issued < nk) {
+          issue(ktBegin + issued, cur); // slab i + NS takes the buffer of slab i
+          issued++;
+        }
         loadFrags((i + 1) % NS, 0, fa[0], fb[0]);
       }
       mfmaStep(fa[(KSTEPS - 1) & 1], fb[(KSTEPS - 1) & 1]);
