@@ -38,6 +38,16 @@ namespace gemmk {
 #define HOM_PIPE_TILE_D HOM_PIPE_TILE_A
 #define HOM_FINE_TILE(BM, BN, WM, WN, DIST)                                    \
   HOM_EXTERN_EPILOGUES(launchFine, BM, BN, WM, WN, DIST)
+#define HOM_EXTERN_Q(E, NK, BM, BN, WM, WN, DIST)                              \
+  extern template Status launchPipe<BM, BN, WM, WN, DIST, E, NK, true>(        \
+      const GemmProblem &, hipStream_t);
+#define HOM_PIPE_TILE_Q(BM, BN, WM, WN, DIST)                                  \
+  HOM_EXTERN_Q(0, false, BM, BN, WM, WN, DIST)                                 \
+  HOM_EXTERN_Q(0, true, BM, BN, WM, WN, DIST)                                  \
+  HOM_EXTERN_Q(1, false, BM, BN, WM, WN, DIST)                                 \
+  HOM_EXTERN_Q(1, true, BM, BN, WM, WN, DIST)                                  \
+  HOM_EXTERN_Q(2, false, BM, BN, WM, WN, DIST)                                 \
+  HOM_EXTERN_Q(2, true, BM, BN, WM, WN, DIST)
 #define HOM_STAGED_TILE(BM, BN, BK, WM, WN, VEC)                               \
   HOM_EXTERN_STAGED(BM, BN, BK, WM, WN, 0, VEC)                                \
   HOM_EXTERN_STAGED(BM, BN, BK, WM, WN, 1, VEC)                                \
@@ -49,6 +59,7 @@ namespace gemmk {
 #undef HOM_PIPE_TILE_C
 #undef HOM_PIPE_TILE_D
 #undef HOM_FINE_TILE
+#undef HOM_PIPE_TILE_Q
 #undef HOM_STAGED_TILE
 } // namespace gemmk
 
@@ -90,6 +101,21 @@ struct KernelEntry {
         launchPipe<BM, BN, WM, WN, DIST, int(EPI_ENUM), false>,                \
         launchPipe<BM, BN, WM, WN, DIST, int(EPI_ENUM), true>                  \
   }
+// "q<d>": the same pipeline with slabs staged by buffer_load ... lds into a
+// ring of d + 1 LDS buffers (d slabs in flight).
+#define HOM_PIPE_Q_ENTRY(BM, BN, WM, WN, DIST, EPI_ENUM, EPI_STR, ACT)         \
+  {                                                                            \
+    {"hom_gfx950_mfma_f16_s32x32x16gemm_f16_" #BM "x" #BN "_64q" #DIST         \
+     "_w" #WM "x" #WN "_nn_align8_" EPI_STR,                                   \
+     BM, BN, 64, WM, WN, 8, 2, ACT, EPI_ENUM},                                 \
+        launchPipe<BM, BN, WM, WN, DIST, int(EPI_ENUM), false, true>,          \
+        launchPipe<BM, BN, WM, WN, DIST, int(EPI_ENUM), true, true>            \
+  }
+#define HOM_PIPE_TILE_Q(BM, BN, WM, WN, DIST)                                  \
+  HOM_PIPE_Q_ENTRY(BM, BN, WM, WN, DIST, Epilogue::kLinear, "linear", 0),      \
+      HOM_PIPE_Q_ENTRY(BM, BN, WM, WN, DIST, Epilogue::kGeluErf, "gelu", 1),   \
+      HOM_PIPE_Q_ENTRY(BM, BN, WM, WN, DIST, Epilogue::kGeluTanh, "gelutanh",  \
+                       1),
 #define HOM_PIPE_TILE_A(BM, BN, WM, WN, DIST)                                  \
   HOM_PIPE_ENTRY(BM, BN, WM, WN, DIST, Epilogue::kLinear, "linear", 0),        \
       HOM_PIPE_ENTRY(BM, BN, WM, WN, DIST, Epilogue::kGeluErf, "gelu", 1),     \

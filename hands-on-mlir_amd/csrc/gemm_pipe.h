@@ -19,7 +19,8 @@ namespace gemmk {
 // memory.  `rest` holds the same values again plus everything else; its copies
 // of the leading arguments are never read.
 // tileWalk = xcdR | lastRows << 4 | fullGroups << 8.
-template <int BM, int BN, int WM, int WN, int DIST, int EPI, bool B_NK>
+template <int BM, int BN, int WM, int WN, int DIST, int EPI, bool B_NK,
+          bool DMA = false>
 __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(
     const _Float16 *argA, const _Float16 *argB, int argM, int argN, int argK,
     int argLda, int argLdb, int argTilesN, int argXcdQ, uint32_t argTileWalk,
@@ -59,6 +60,12 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(
   constexpr int B_ROW_BYTES = B_NK ? 128 : BN * 2;
   constexpr int B_VPR = B_ROW_BYTES / 16; // vectors per LDS row of B
   constexpr int KSTEPS = BK / 16;
+  // DMA: slabs travel global memory -> LDS without passing through registers
+  // (buffer_load ... lds), into a ring of DIST + 1 buffers: the slab being
+  // multiplied and DIST slabs landed or on their way.  An LDS write from
+  // registers moves 75 bytes per clock and CU and takes the LDS pipe from the
+  // fragment reads; the DMA path leaves it to them.
+  constexpr int NBUF = DMA ? DIST + 1 : 2;
   // Tiles up to 128 x 128 serve problems of a few microseconds, where the way
   // to the first memory request and back counts as much as the main loop;
   // larger tiles keep the order that suits their register budget.
@@ -152,51 +159,80 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(
   int aDst0 = 0, bDst0 = 0;
   int aK[A_PER_T], bK[B_PER_T]; // k position inside the slab
 #pragma unroll
+  // DMA: a wavefront's instruction fills 1 KiB of LDS in lane order, so vector v
+  // lands at byte 16 v and the swizzle is applied on the source side: the lane
+  // fetches the chunk that belongs at its position.
   for (int i = 0; i < A_PER_T; i++) {
     const int v = tid + i * THREADS;
-    const int r = v / 8, c = v % 8;
+    const int r = v / 8, c = DMA ? swzK(r, v % 8) : v % 8;
     aK[i] = c * 8;
     aOff[i] = (uint32_t(r) * uint32_t(p.lda) + c * 8) * 2u;
     if (i == 0)
-      aDst0 = r * 128 + swzK(r, c) * 16;
+      aDst0 = DMA ? v * 16 : r * 128 + swzK(r, c) * 16;
   }
 #pragma unroll
   for (int i = 0; i < B_PER_T; i++) {
     const int v = tid + i * THREADS;
-    const int r = v / B_VPR, c = v % B_VPR;
+    const int r = v / B_VPR, pc = v % B_VPR;
     if (B_NK) {
+      const int c = DMA ? swzK(r, pc) : pc;
       bK[i] = c * 8;
       bOff[i] = (uint32_t(r) * uint32_t(p.ldb) + c * 8) * 2u;
       if (i == 0)
-        bDst0 = r * 128 + swzK(r, c) * 16;
+        bDst0 = DMA ? v * 16 : r * 128 + swzK(r, c) * 16;
     } else {
+      const int c = DMA ? swzN<BN>(r, pc / 4) * 4 + pc % 4 : pc;
       bK[i] = r;
       bOff[i] = (uint32_t(r) * uint32_t(p.ldb) + c * 8) * 2u;
       if (i == 0)
-        bDst0 = r * B_ROW_BYTES + swzN<BN>(r, c / 4) * 64 + (c % 4) * 16;
+        bDst0 = DMA ? v * 16
+                    : r * B_ROW_BYTES + swzN<BN>(r, c / 4) * 64 + (c % 4) * 16;
     }
   }
 
-  half8 regA[DIST][A_PER_T], regB[DIST][B_PER_T];
+  half8 regA[DMA ? 1 : DIST][A_PER_T], regB[DMA ? 1 : DIST][B_PER_T];
   // Slabs of this slice that lie inside [0, kEnd) entirely, and whether a
   // partial one follows them (only the last slice of a ragged K has one).
   const int nkFull = (kEnd - ktBegin * BK) / BK;
   const bool hasTail = kEnd - ktBegin * BK > nkFull * BK;
   const int ktLastFull = ktBegin + nkFull - 1;
   // Full slab kt (requests past the last full slab fetch that one again).
+  // One vector of a full slab straight into LDS buffer `stage` (DMA).
+  auto dmaVec = [&](int stage, int k0, auto vC) {
+#if defined(__HIP_DEVICE_COMPILE__) // (the builtin's LDS pointer type exists only for the GPU target)
+    constexpr int V = decltype(vC)::value;
+    unsigned char *st = smem + stage * STAGE_BYTES;
+    if constexpr (V < A_PER_T) {
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(
+          rsrcA, HOM_LDS_PTR(st + (V * THREADS + wave * kWave) * 16), 16,
+          aOff[V], uint32_t(k0) * 2u, 0, 0);
+    } else {
+      constexpr int W = V - A_PER_T;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(
+          rsrcB, HOM_LDS_PTR(st + A_BYTES + (W * THREADS + wave * kWave) * 16),
+          16, bOff[W],
+          B_NK ? uint32_t(k0) * 2u : uint32_t(k0) * uint32_t(p.ldb) * 2u, 0, 0);
+    }
+#endif
+  };
   auto loadGlobal = [&](int kt, auto setC) {
     constexpr int S = decltype(setC)::value;
     const int k0 = (kt < ktLastFull ? kt : ktLastFull) * BK;
-    const uint32_t sA = uint32_t(k0) * 2u;
-    const uint32_t sB = B_NK ? sA : uint32_t(k0) * uint32_t(p.ldb) * 2u;
+    if constexpr (DMA) {
+      // (set S: the slab goes to ring buffer S)
+      staticFor<A_PER_T + B_PER_T>([&](auto vC) { dmaVec(S, k0, vC); });
+    } else {
+      const uint32_t sA = uint32_t(k0) * 2u;
+      const uint32_t sB = B_NK ? sA : uint32_t(k0) * uint32_t(p.ldb) * 2u;
 #pragma unroll
-    for (int i = 0; i < A_PER_T; i++)
-      regA[S][i] = __builtin_bit_cast(
-          half8, __builtin_amdgcn_raw_buffer_load_b128(rsrcA, aOff[i], sA, 0));
+      for (int i = 0; i < A_PER_T; i++)
+        regA[S][i] = __builtin_bit_cast(
+            half8, __builtin_amdgcn_raw_buffer_load_b128(rsrcA, aOff[i], sA, 0));
 #pragma unroll
-    for (int i = 0; i < B_PER_T; i++)
-      regB[S][i] = __builtin_bit_cast(
-          half8, __builtin_amdgcn_raw_buffer_load_b128(rsrcB, bOff[i], sB, 0));
+      for (int i = 0; i < B_PER_T; i++)
+        regB[S][i] = __builtin_bit_cast(
+            half8, __builtin_amdgcn_raw_buffer_load_b128(rsrcB, bOff[i], sB, 0));
+    }
   };
   // Slab kt with a range test per vector (the partial slab).
   auto loadGlobalChecked = [&](int kt, auto setC) {
@@ -289,6 +325,15 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(
                 swzN<BN>(trRow, group) * 64 + trCol * 2;
   }
 
+  // Fragment registers: one set per k step parity, or one per k step of a slab
+  // (kWholeSlabFrags, see the main loop).  DMA with a row-major B keeps the two
+  // halves of a transposed fragment apart until tieFragments() has waited for
+  // them.
+  constexpr bool kWholeSlabFrags = MI * NI == 1;
+  constexpr int FSETS = kWholeSlabFrags ? KSTEPS : 2;
+  half8 fa[FSETS][MI], fb[FSETS][NI];
+  half8(*const fbSets)[NI] = fb;
+  short4v fbHalf[DMA && !B_NK ? FSETS : 1][NI][2];
   // One fragment per call: unit u < MI is A block u, the rest are B blocks.
   auto loadFragUnit = [&](int stage, int kk, half8 (&fa)[MI], half8 (&fb)[NI],
                           auto uC) {
@@ -301,20 +346,37 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(
       fb[j] = *reinterpret_cast<const half8 *>(st + bFragK[kk] + j * 32 * 128);
     } else {
       constexpr int j = U - MI;
-      short4v t[2];
+      if constexpr (DMA) {
+        // Issued behind the compiler's back: it would put a wait for every
+        // outstanding DMA load in front of a transposing read (it cannot tell
+        // that the read's buffer is not one a load is filling).  The halves
+        // are put together, behind a wait, by tieFragments().
+        const int set = int(&fb - fbSets);
+        const uint32_t at = uint32_t(uintptr_t(HOM_LDS_PTR(st + bFragN[j])));
 #pragma unroll
-      for (int h = 0; h < 2; h++)
-        t[h] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-            (__attribute__((address_space(3))) short4v *)(
-                st + bFragN[j] + (kk * 16 + h * 4) * B_ROW_BYTES));
-      typedef short short8v __attribute__((ext_vector_type(8)));
-      short8v both;
+        for (int h = 0; h < 2; h++) {
+          short4v half;
+          asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2"
+                       : "=v"(half)
+                       : "v"(at), "i"((kk * 16 + h * 4) * B_ROW_BYTES));
+          fbHalf[set][j][h] = half;
+        }
+      } else {
+        short4v t[2];
 #pragma unroll
-      for (int e = 0; e < 4; e++) {
-        both[e] = t[0][e];
-        both[4 + e] = t[1][e];
+        for (int h = 0; h < 2; h++)
+          t[h] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+              (__attribute__((address_space(3))) short4v *)(
+                  st + bFragN[j] + (kk * 16 + h * 4) * B_ROW_BYTES));
+        typedef short short8v __attribute__((ext_vector_type(8)));
+        short8v both;
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          both[e] = t[0][e];
+          both[4 + e] = t[1][e];
+        }
+        fb[j] = __builtin_bit_cast(half8, both);
       }
-      fb[j] = __builtin_bit_cast(half8, both);
     }
   };
   auto loadFrags = [&](int stage, int kk, half8 (&fa)[MI], half8 (&fb)[NI]) {
@@ -346,9 +408,6 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(
   // of a slab's fragments requested at once behind the barrier, a slab exposes
   // one round trip: 1024x768x3072 13.4 -> 12.7 us, 1024x768x768 5.5 -> 5.3 us.
   // (Two blocks per wave tile, 128x128 with 2x4 wavefronts: 2 % slower.)
-  constexpr bool kWholeSlabFrags = MI * NI == 1;
-  constexpr int FSETS = kWholeSlabFrags ? KSTEPS : 2;
-  half8 fa[FSETS][MI], fb[FSETS][NI];
   const int nk = nkFull; // the pipelined loop walks the full slabs
   // Moves vector v of register set S to LDS and refills it from full slab kt
   // (already clamped to the last full slab by the caller).
@@ -358,7 +417,9 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(
     unsigned char *sA = smem + stage * STAGE_BYTES;
     unsigned char *sB = sA + A_BYTES;
     const int k0 = kt * BK;
-    if constexpr (V < A_PER_T) {
+    if constexpr (DMA) {
+      dmaVec(stage, k0, vC);
+    } else if constexpr (V < A_PER_T) {
       *reinterpret_cast<half8 *>(sA + aDst0 + V * DST_STEP) = regA[S][V];
       regA[S][V] = __builtin_bit_cast(
           half8, __builtin_amdgcn_raw_buffer_load_b128(rsrcA, aOff[V],
@@ -374,6 +435,28 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(
               0));
     }
   };
+  // Row-major B staged by DMA: the transposing reads were issued by hand, so
+  // the wait for them is by hand as well, and the fragments pass through it so
+  // that no MFMA on them can be moved in front of it.
+  auto tieFragments = [&](half8 (&b)[NI]) {
+    if constexpr (DMA && !B_NK) {
+      const int set = int(&b - fbSets);
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      staticFor<NI>([&](auto jC) {
+        constexpr int j = decltype(jC)::value;
+        short4v lo = fbHalf[set][j][0], hi = fbHalf[set][j][1];
+        asm volatile("" : "+v"(lo), "+v"(hi)); // not before the wait
+        typedef short short8v __attribute__((ext_vector_type(8)));
+        short8v both;
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          both[e] = lo[e];
+          both[4 + e] = hi[e];
+        }
+        b[j] = __builtin_bit_cast(half8, both);
+      });
+    }
+  };
   // The MFMAs of one k step on fragments (a, b).  Spread between them: the
   // fragment reads of another k step (rdStage, rdKk) into (na, nb) when RD, and
   // the staging vectors [V0, V1) when stageOn.  Memory operation q of n goes in
@@ -386,6 +469,7 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(
     constexpr int V0 = decltype(v0C)::value, V1 = decltype(v1C)::value;
     constexpr int NR = RD ? MI + NI : 0;
     constexpr int N = NR + (V1 - V0);
+    tieFragments(b);
     staticFor<NM>([&](auto mC) {
       constexpr int m = decltype(mC)::value;
       if constexpr (N > 0) {
@@ -410,13 +494,31 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(
     });
     __builtin_amdgcn_sched_barrier(0);
   };
+  // The barrier between slab i and slab i+1: every wavefront has its last
+  // fragments of slab i, and slab i+1 is complete in its buffer.  DMA: a
+  // wavefront's loads land in the order it issued them, NV per slab, and slabs
+  // up to i+DIST have been issued, so slab i+1 is there when at most
+  // (DIST-1) * NV loads are outstanding.
+  auto slabBarrier = [&]() {
+    if constexpr (DMA)
+      asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(
+                       (DIST - 1) * NV)
+                   : "memory");
+    else
+      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+  };
   // tailC: the slab may be the last one (then nothing follows it); the
   // steady-state loop knows it is not and runs without branches.
   auto slab = [&](int i, auto setC, auto tailC) {
     constexpr bool kTail = decltype(tailC)::value;
-    const int cur = i & 1;
+    // Register staging: slab i+1 moves from its registers to the other buffer
+    // and the registers are refilled with slab i+1+DIST.  DMA: the buffer that
+    // slab i-1 left takes slab i+DIST.
+    const int cur = DMA ? i % NBUF : i & 1;
+    const int nxt = DMA ? (i + 1) % NBUF : cur ^ 1;
+    const int fill = DMA ? (i + DIST) % NBUF : cur ^ 1;
     const bool more = !kTail || i + 1 < nk;
-    const int ktWant = ktBegin + i + 1 + DIST;
+    const int ktWant = ktBegin + i + DIST + (DMA ? 0 : 1);
     const int ktNext = ktWant < ktLastFull ? ktWant : ktLastFull;
     staticFor<KSTEPS>([&](auto kkC) {
       constexpr int kk = decltype(kkC)::value;
@@ -427,15 +529,15 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(
       constexpr int cs = kk % 2, ns = (kk + 1) % 2;
       if constexpr (kk < KSTEPS - 1) {
         mfmaMixed(fa[cs], fb[cs], fa[ns], fb[ns], cur, kk + 1, std::true_type{},
-                  cur ^ 1, ktNext, more, setC, V0C{}, V1C{});
+                  fill, ktNext, more, setC, V0C{}, V1C{});
       } else {
         static_assert(ns == 0, "the next slab finds its first fragments in set 0");
         if (more) {
           // Every wavefront has its last fragments of slab i in registers and
           // slab i+1 is complete in the other buffer after this barrier; its
           // first fragments arrive under the MFMAs of the last k step.
-          asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-          mfmaMixed(fa[cs], fb[cs], fa[ns], fb[ns], cur ^ 1, 0, std::true_type{},
+          slabBarrier();
+          mfmaMixed(fa[cs], fb[cs], fa[ns], fb[ns], nxt, 0, std::true_type{},
                     0, 0, false, setC, V0C{}, V1C{});
         } else {
           mfmaMixed(fa[cs], fb[cs], fa[ns], fb[ns], 0, 0, std::false_type{}, 0,
@@ -452,9 +554,11 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(
   // and the last set is requested again.
   auto slabWhole = [&](int i, auto setC, auto tailC) {
     constexpr bool kTail = decltype(tailC)::value;
-    const int cur = i & 1;
+    const int cur = DMA ? i % NBUF : i & 1;
+    const int nxt = DMA ? (i + 1) % NBUF : cur ^ 1;
+    const int fill = DMA ? (i + DIST) % NBUF : cur ^ 1;
     const bool more = !kTail || i + 1 < nk;
-    const int ktWant = ktBegin + i + 1 + DIST;
+    const int ktWant = ktBegin + i + DIST + (DMA ? 0 : 1);
     const int ktNext = ktWant < ktLastFull ? ktWant : ktLastFull;
     staticFor<KSTEPS - 1>([&](auto kkC) {
       constexpr int kk = decltype(kkC)::value;
@@ -463,28 +567,30 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(
       using V1C = std::integral_constant<int, V1>;
       constexpr int fs = kk % FSETS;
       mfmaMixed(fa[fs], fb[fs], fa[fs], fb[fs], 0, 0, std::false_type{},
-                cur ^ 1, ktNext, more, setC, V0C{}, V1C{});
+                fill, ktNext, more, setC, V0C{}, V1C{});
     });
     constexpr int last = (KSTEPS - 1) % FSETS;
     using VE = std::integral_constant<int, NV>;
     if (more) {
-      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+      slabBarrier();
       staticFor<KSTEPS - 1>([&](auto kkC) {
         constexpr int kk = decltype(kkC)::value;
-        loadFrags(cur ^ 1, kk, fa[kk % FSETS], fb[kk % FSETS]);
+        loadFrags(nxt, kk, fa[kk % FSETS], fb[kk % FSETS]);
       });
       __builtin_amdgcn_sched_barrier(0);
     }
     mfmaMixed(fa[last], fb[last], fa[last], fb[last], 0, 0, std::false_type{},
               0, 0, false, setC, VE{}, VE{});
     if (more) {
-      loadFrags(cur ^ 1, KSTEPS - 1, fa[last], fb[last]);
+      loadFrags(nxt, KSTEPS - 1, fa[last], fb[last]);
       __builtin_amdgcn_sched_barrier(0);
     }
   };
   // The partial slab of a ragged K, unpipelined: one slab of the whole problem.
   auto raggedSlab = [&]() {
     using Set0 = std::integral_constant<int, 0>;
+    if constexpr (DMA) // nothing may still be on its way into buffer 0
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     loadGlobalChecked(ktBegin + nkFull, Set0{});
     __syncthreads(); // no wavefront still reads a full slab from buffer 0
     storeLds(0, Set0{});
@@ -492,6 +598,7 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(
 #pragma unroll
     for (int kk = 0; kk < KSTEPS; kk++) {
       loadFrags(0, kk, fa[0], fb[0]);
+      tieFragments(fb[0]);
 #pragma unroll
       for (int m = 0; m < NM; m++)
         acc[m / NI][m % NI] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
@@ -507,9 +614,16 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(
     if constexpr (!kLatencyFirst)
       staticFor<DIST>(
           [&](auto d) { loadGlobal(ktBegin + decltype(d)::value, d); });
-    storeLds(0, std::integral_constant<int, 0>{});
-    loadGlobal(ktBegin + DIST, std::integral_constant<int, 0>{});
-    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    if constexpr (DMA) {
+      // slabs 0 .. DIST-1 are on their way to buffers 0 .. DIST-1; slab 0 has
+      // landed when the DIST-1 slabs behind it are all that is outstanding
+      asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"((DIST - 1) * NV)
+                   : "memory");
+    } else {
+      storeLds(0, std::integral_constant<int, 0>{});
+      loadGlobal(ktBegin + DIST, std::integral_constant<int, 0>{});
+      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    }
     if constexpr (kWholeSlabFrags) {
       staticFor<KSTEPS>([&](auto kkC) {
         constexpr int kk = decltype(kkC)::value;
@@ -545,8 +659,10 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(
     if (hasTail)
       raggedSlab(); // behind the full slabs, whose requests went out first
   }
+  if constexpr (DMA) // the ring's last requests (never read) land before LDS is reused
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
-  static_assert(WM * WN * 32 * (WTN * 4 + 16) <= 2 * STAGE_BYTES,
+  static_assert(WM * WN * 32 * (WTN * 4 + 16) <= NBUF * STAGE_BYTES,
                 "epilogue strips must fit the main loop's LDS");
   if (numSlices > 1)
     storePartial<MI, NI, THREADS>(p, acc, tile, slice, numSlices, tid);
@@ -557,9 +673,14 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(
   } while (vpid < nTiles); // tiles of this workgroup
 }
 
-template <int BM, int BN, int WM, int WN, int DIST, int EPI, bool B_NK>
+template <int BM, int BN, int WM, int WN, int DIST, int EPI, bool B_NK,
+          bool DMA = false>
 Status launchPipe(const GemmProblem &pr, hipStream_t s) {
-  constexpr int SMEM = 2 * (BM + BN) * 64 * 2;
+  constexpr int SMEM = (DMA ? DIST + 1 : 2) * (BM + BN) * 64 * 2;
+  static_assert(!DMA || ((BM * 8) % (WM * WN * kWave) == 0 &&
+                         (BN * 8) % (WM * WN * kWave) == 0 &&
+                         (B_NK || 1024 % (BN * 2) == 0 || (BN * 2) % 1024 == 0)),
+                "a DMA instruction fills 1 KiB: whole rows of the tile");
   LaunchPlan plan;
   Status st = planLaunch<BM, BN, 64>(pr, &plan);
   if (st != Status::kSuccess)
@@ -571,7 +692,7 @@ Status launchPipe(const GemmProblem &pr, hipStream_t s) {
   HOM_CHECK_RET((int64_t(BM) * pr.lda + pr.K) * 2 < (int64_t(1) << 31) &&
                     (int64_t(BN) * pr.ldb + pr.K) * 2 < (int64_t(1) << 31),
                 Status::kInvalidArgument, "gemm: leading dimension too large");
-  auto kernel = gemmPipeKernel<BM, BN, WM, WN, DIST, EPI, B_NK>;
+  auto kernel = gemmPipeKernel<BM, BN, WM, WN, DIST, EPI, B_NK, DMA>;
   static bool attrSet = false;
   st = allowLds(kernel, SMEM, &attrSet);
   if (st != Status::kSuccess)

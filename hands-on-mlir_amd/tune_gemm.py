@@ -38,8 +38,11 @@ def bert_shapes():
     return shapes
 
 
-TILES = [(64, 64, 2, 2, 2), (64, 64, 2, 2, 4), (128, 64, 2, 2, 2), (64, 128, 2, 2, 2), (128, 128, 2, 4, 2),
-         (128, 256, 2, 4, 2), (256, 128, 4, 2, 2), (256, 256, 2, 4, 1), (128, 96, 4, 1, 2), (256, 96, 4, 1, 2)]
+# (BM, BN, WM, WN, slabs in flight, staging: "x2r" registers + 2 LDS buffers, "q" buffer_load ... lds into a ring)
+TILES = [(64, 64, 2, 2, 2, "x2r"), (64, 64, 2, 2, 4, "x2r"), (128, 64, 2, 2, 2, "x2r"), (64, 128, 2, 2, 2, "x2r"),
+         (128, 128, 2, 4, 2, "x2r"), (128, 256, 2, 4, 2, "x2r"), (256, 128, 4, 2, 2, "x2r"), (256, 256, 2, 4, 1, "x2r"),
+         (128, 96, 4, 1, 2, "x2r"), (256, 96, 4, 1, 2, "x2r"),
+         (128, 128, 2, 4, 2, "q"), (128, 128, 2, 4, 3, "q"), (64, 64, 2, 2, 3, "q"), (256, 256, 2, 4, 1, "q")]
 
 
 class Row:
@@ -95,8 +98,8 @@ def in_graph_pass(rt, table):
                 start = enc.gemm_choices()[role]
                 best_us, best = forward_us(enc), None
                 epi = "gelu" if key[3] == 1 else "linear"
-                for (bm, bn, wm, wn, depth) in TILES:
-                    name = (f"hom_gfx950_mfma_f16_s32x32x16gemm_f16_{bm}x{bn}_64x2r{depth}_w{wm}x{wn}"
+                for (bm, bn, wm, wn, depth, staging) in TILES:
+                    name = (f"hom_gfx950_mfma_f16_s32x32x16gemm_f16_{bm}x{bn}_64{staging}{depth}_w{wm}x{wn}"
                             f"_nn_align8_{epi}")
                     if number[name] == start[0]:
                         continue
