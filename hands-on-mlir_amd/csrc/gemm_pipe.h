@@ -332,6 +332,7 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(
   constexpr bool kWholeSlabFrags = MI * NI == 1;
   constexpr int FSETS = kWholeSlabFrags ? KSTEPS : 2;
   half8 fa[FSETS][MI], fb[FSETS][NI];
+  constexpr bool kHandReads = DMA && !B_NK;
   half8(*const fbSets)[NI] = fb;
   short4v fbHalf[DMA && !B_NK ? FSETS : 1][NI][2];
   // One fragment per call: unit u < MI is A block u, the rest are B blocks.
@@ -339,7 +340,16 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(
                           auto uC) {
     constexpr int U = decltype(uC)::value;
     const unsigned char *st = smem + stage * STAGE_BYTES;
-    if constexpr (U < MI) {
+    if constexpr (U < MI && kHandReads) {
+      // (see the B units below: in this mode every fragment read is issued
+      // and waited for by hand, so that the waits can be exact)
+      const uint32_t at = uint32_t(uintptr_t(HOM_LDS_PTR(st + aFrag[kk])));
+      half8 frag;
+      asm volatile("ds_read_b128 %0, %1 offset:%2"
+                   : "=v"(frag)
+                   : "v"(at), "i"(U * 32 * 128));
+      fa[U] = frag;
+    } else if constexpr (U < MI) {
       fa[U] = *reinterpret_cast<const half8 *>(st + aFrag[kk] + U * 32 * 128);
     } else if constexpr (B_NK) {
       constexpr int j = U - MI;
@@ -349,8 +359,11 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(
       if constexpr (DMA) {
         // Issued behind the compiler's back: it would put a wait for every
         // outstanding DMA load in front of a transposing read (it cannot tell
-        // that the read's buffer is not one a load is filling).  The halves
-        // are put together, behind a wait, by tieFragments().
+        // that the read's buffer is not one a load is filling).  The compiler
+        // does not count reads it cannot see, so its waits for the reads it
+        // can see would come out stricter than needed; hence all of them by
+        // hand.  The halves are put together, behind a wait, by
+        // tieFragments().
         const int set = int(&fb - fbSets);
         const uint32_t at = uint32_t(uintptr_t(HOM_LDS_PTR(st + bFragN[j])));
 #pragma unroll
@@ -438,10 +451,24 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(
   // Row-major B staged by DMA: the transposing reads were issued by hand, so
   // the wait for them is by hand as well, and the fragments pass through it so
   // that no MFMA on them can be moved in front of it.
-  auto tieFragments = [&](half8 (&b)[NI]) {
-    if constexpr (DMA && !B_NK) {
+  // Hand-issued fragment reads (kHandReads): the wait for the fragments of a k
+  // step, and the fragments pass through it so that no MFMA on them can be
+  // moved in front of it.  allowC: how many LDS reads were issued after the
+  // last one of this k step (they may stay outstanding; LDS reads return in
+  // order); negative: the caller has waited.
+  using TieNow = std::integral_constant<int, 0>;
+  auto tieFragments = [&](half8 (&a)[MI], half8 (&b)[NI], auto allowC) {
+    constexpr int kAllow = decltype(allowC)::value;
+    if constexpr (kHandReads) {
       const int set = int(&b - fbSets);
-      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      if constexpr (kAllow >= 0)
+        asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(kAllow < 15 ? kAllow : 15)
+                     : "memory");
+      staticFor<MI>([&](auto iC) {
+        half8 frag = a[decltype(iC)::value];
+        asm volatile("" : "+v"(frag)); // not before the wait
+        a[decltype(iC)::value] = frag;
+      });
       staticFor<NI>([&](auto jC) {
         constexpr int j = decltype(jC)::value;
         short4v lo = fbHalf[set][j][0], hi = fbHalf[set][j][1];
@@ -464,12 +491,12 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(
   auto mfmaMixed = [&](half8 (&a)[MI], half8 (&b)[NI], half8 (&na)[MI],
                        half8 (&nb)[NI], int rdStage, int rdKk, auto rdC,
                        int stStage, int kt, bool stageOn, auto setC, auto v0C,
-                       auto v1C) {
+                       auto v1C, auto allowC) {
     constexpr bool RD = decltype(rdC)::value;
     constexpr int V0 = decltype(v0C)::value, V1 = decltype(v1C)::value;
     constexpr int NR = RD ? MI + NI : 0;
     constexpr int N = NR + (V1 - V0);
-    tieFragments(b);
+    tieFragments(a, b, allowC);
     staticFor<NM>([&](auto mC) {
       constexpr int m = decltype(mC)::value;
       if constexpr (N > 0) {
@@ -529,7 +556,7 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(
       constexpr int cs = kk % 2, ns = (kk + 1) % 2;
       if constexpr (kk < KSTEPS - 1) {
         mfmaMixed(fa[cs], fb[cs], fa[ns], fb[ns], cur, kk + 1, std::true_type{},
-                  fill, ktNext, more, setC, V0C{}, V1C{});
+                  fill, ktNext, more, setC, V0C{}, V1C{}, TieNow{});
       } else {
         static_assert(ns == 0, "the next slab finds its first fragments in set 0");
         if (more) {
@@ -538,10 +565,10 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(
           // first fragments arrive under the MFMAs of the last k step.
           slabBarrier();
           mfmaMixed(fa[cs], fb[cs], fa[ns], fb[ns], nxt, 0, std::true_type{},
-                    0, 0, false, setC, V0C{}, V1C{});
+                    0, 0, false, setC, V0C{}, V1C{}, TieNow{});
         } else {
           mfmaMixed(fa[cs], fb[cs], fa[ns], fb[ns], 0, 0, std::false_type{}, 0,
-                    0, false, setC, V0C{}, V1C{});
+                    0, false, setC, V0C{}, V1C{}, TieNow{});
         }
       }
     });
@@ -566,8 +593,11 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(
       using V0C = std::integral_constant<int, V0>;
       using V1C = std::integral_constant<int, V1>;
       constexpr int fs = kk % FSETS;
+      // the fragments of the later k steps were requested behind these
       mfmaMixed(fa[fs], fb[fs], fa[fs], fb[fs], 0, 0, std::false_type{},
-                fill, ktNext, more, setC, V0C{}, V1C{});
+                fill, ktNext, more, setC, V0C{}, V1C{},
+                std::integral_constant<int, (KSTEPS - 1 - kk) *
+                                                (MI + 2 * NI)>{});
     });
     constexpr int last = (KSTEPS - 1) % FSETS;
     using VE = std::integral_constant<int, NV>;
@@ -578,9 +608,13 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(
         loadFrags(nxt, kk, fa[kk % FSETS], fb[kk % FSETS]);
       });
       __builtin_amdgcn_sched_barrier(0);
+      // the barrier's wait covered the last k step's fragments
+      tieFragments(fa[last], fb[last], std::integral_constant<int, 15>{});
+    } else {
+      tieFragments(fa[last], fb[last], TieNow{});
     }
     mfmaMixed(fa[last], fb[last], fa[last], fb[last], 0, 0, std::false_type{},
-              0, 0, false, setC, VE{}, VE{});
+              0, 0, false, setC, VE{}, VE{}, std::integral_constant<int, -1>{});
     if (more) {
       loadFrags(nxt, KSTEPS - 1, fa[last], fb[last]);
       __builtin_amdgcn_sched_barrier(0);
@@ -598,7 +632,7 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(
 #pragma unroll
     for (int kk = 0; kk < KSTEPS; kk++) {
       loadFrags(0, kk, fa[0], fb[0]);
-      tieFragments(fb[0]);
+      tieFragments(fa[0], fb[0], TieNow{});
 #pragma unroll
       for (int m = 0; m < NM; m++)
         acc[m / NI][m % NI] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
