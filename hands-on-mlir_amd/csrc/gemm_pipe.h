@@ -6,12 +6,16 @@ namespace hom {
 namespace gemmk {
 
 // ==================================================================== pipe ==
-// Same LDS layout, fragment reads and barrier placement as the dma kernels, but
-// the slabs travel global -> registers -> LDS (two LDS buffers): the loads of
-// slab i+1 are issued before slab i is multiplied and written to LDS after it.
-// The vector memory path into registers sustains several times the bandwidth
-// of the LDS-DMA path on this chip, which matters once a CU streams more than
-// ~16 bytes per clock (large tiles, or several workgroups per CU).
+// Same LDS layout, fragment reads and barrier placement as the dma kernels.
+// DMA == false: the slabs travel global -> registers -> LDS (two LDS buffers);
+// the loads of slab i+1 are issued before slab i is multiplied and written to
+// LDS after it, DIST slabs are in flight in registers.  DMA == true: the same
+// pipeline with buffer_load ... lds into a ring of DIST + 1 LDS buffers, which
+// takes the staging writes (75 bytes per clock and CU when issued from
+// registers, a third of the read rate) off the LDS pipe the fragment reads
+// need.  Both stage at the rate the L1 delivers (about 50 bytes per clock and
+// CU); the DMA variant is 1.5-8 % faster at M = 1024 and equal for 256 x 256
+// tiles, where only one slab in flight fits in LDS.
 // What the kernel needs on its way to the first loads travels as leading
 // scalar arguments (14 dwords): the command processor delivers those in scalar
 // registers when the wavefront starts (kernel-argument preload, see the
