@@ -189,13 +189,18 @@ def test_gemm_every_manifest_kernel(gpu, rt, oracle):
 FINE_TILES = ("128x96_64x2r2_w4x2", "64x48_64x2r2_w4x1", "64x48_64x2r4_w4x1", "64x144_64x2r2_w4x1")
 
 
-def test_gemm_fine_family(gpu, rt, oracle, monkeypatch):
-    """The 16x16x32-MFMA kernels (tile sides in steps of 16): every epilogue source form (none, bias row,
-    in-place residual, a [M', N] source shared by the batch entries = the general epilogue), GELU, split-K,
-    ragged M / N / K, more tiles than CUs, and the [N, K] layout of B through nvteGemmF16."""
-    g = np.random.default_rng(41)
+# the register-staged pipeline with slabs staged by buffer_load ... lds (ring of LDS buffers, fragment reads issued
+# by hand when B is row-major)
+DMA_STAGED_TILES = ("128x128_64q2_w2x4", "128x128_64q3_w2x4", "64x64_64q3_w2x2", "256x256_64q1_w2x4")
+
+
+def _gemm_family_cases(gpu, rt, oracle, monkeypatch, tiles, seed):
+    """Every epilogue source form (none, bias row, in-place residual, a [M', N] source shared by the batch entries
+    = the general epilogue), GELU, split-K, ragged M / N / K (a partial last slab, K smaller than the pipeline is
+    deep), more tiles than CUs, and the [N, K] layout of B through nvteGemmF16."""
+    g = np.random.default_rng(seed)
     M = rt.MemRef.from_tensor
-    for tile in FINE_TILES:
+    for tile in tiles:
         for (M_, N_, K_) in [(256, 288, 128), (200, 264, 136), (72, 40, 392), (1100, 2000, 72)]:
             A = g.standard_normal((1, M_, K_)).astype(np.float16)
             B = (g.standard_normal((1, K_, N_)) * 0.1).astype(np.float16)
@@ -232,6 +237,17 @@ def test_gemm_fine_family(gpu, rt, oracle, monkeypatch):
         monkeypatch.delenv("HOM_NVTE_GEMM_KERNEL")
 
 
+def test_gemm_fine_family(gpu, rt, oracle, monkeypatch):
+    """The 16x16x32-MFMA kernels (tile sides in steps of 16)."""
+    _gemm_family_cases(gpu, rt, oracle, monkeypatch, FINE_TILES, 41)
+
+
+def test_gemm_dma_staged_family(gpu, rt, oracle, monkeypatch):
+    """The q<d> kernels: same cases; K = 72 and 128 are shorter than the ring is deep, 136 and 392 end in a partial
+    slab, 1100 x 2000 has more tiles than the chip holds workgroups."""
+    _gemm_family_cases(gpu, rt, oracle, monkeypatch, DMA_STAGED_TILES, 43)
+
+
 def test_gemm_more_tiles_than_resident_workgroups(gpu, rt, oracle):
     """Ragged problem whose tile count exceeds what the chip holds at once, so the
     persistent kernels walk several tiles per workgroup (with and without split-K)."""
@@ -241,7 +257,8 @@ def test_gemm_more_tiles_than_resident_workgroups(gpu, rt, oracle):
     B = (g.standard_normal((1, K_, N_)) * 0.1).astype(np.float16)
     bias = g.standard_normal((1, 1, N_)).astype(np.float16)
     want = oracle.gemm(A[0], B[0], bias[0], beta=1.0, act="gelu_erf")
-    for tile in ("64x64_64x2r2_w2x2", "128x128_64x2r2_w2x4", "256x256_64x2r1_w2x4"):
+    for tile in ("64x64_64x2r2_w2x2", "128x128_64x2r2_w2x4", "256x256_64x2r1_w2x4", "64x64_64q3_w2x2",
+                 "256x256_64q1_w2x4"):
         for sk in (1, 2):
             got = run_gemm(gpu, rt, A, B, bias, np.zeros((1, M_, N_), np.float16), knum(rt, tile, "gelu"), sk,
                            beta=1.0)
