@@ -4,6 +4,7 @@
 
 what:  gemm1      FFN1 GEMM + bias + tanh-GELU, M=1024 K=768 N=3072 (tuned kernel)
        gemm5      BERT-large FFN2 GEMM, M=16384 K=4096 N=1024
+       gemm5g     BERT-large FFN1 GEMM + bias + erf-GELU, M=16384 K=1024 N=4096
        layernorm  in-place layer norm, 16384 x 1024
        attention  packed-QKV attention, b8 s128 h12
        attention5 packed-QKV attention, b32 s512 h16, full-length sequences
@@ -37,6 +38,10 @@ def main():
         lib.homGemmSelect(16384, 1024, 4096, 0, ctypes.byref(idx), ctypes.byref(sk))
         ms = drv.homTimeGemm(16384, 1024, 4096, 0, 0, idx.value + 1, sk.value, iters, 3)
         print(f"gemm5 {lib.homGemmManifestName(idx.value).decode()} splitK {sk.value}: {ms * 1e3:.2f} us")
+    elif what == "gemm5g":
+        lib.homGemmSelect(16384, 4096, 1024, 1, ctypes.byref(idx), ctypes.byref(sk))
+        ms = drv.homTimeGemm(16384, 4096, 1024, 1, 1, idx.value + 1, sk.value, iters, 3)
+        print(f"gemm5g {lib.homGemmManifestName(idx.value).decode()} splitK {sk.value}: {ms * 1e3:.2f} us")
     elif what == "layernorm":
         print(f"layernorm 16384x1024: {drv.homTimeLayernorm(16384, 1024, 0, iters, 3) * 1e3:.2f} us")
     elif what == "attention":
