@@ -23,7 +23,9 @@ class BertEncoder:
             layout[self.ROLES.index(role)] = {"kn": 0, "nk": 1}[lay]
         self.h = self.drv.homBertCreateWithLayout(layers, hidden, heads, ffn, bs, seq, vocab, gemm_mode,
                                                   1 if gelu_form == "tanh" else 0, layout)
-        assert self.h, "homBertCreate failed"
+        if not self.h:
+            raise ValueError("homBertCreateWithLayout refused the configuration (a GELU role of an erf-GELU "
+                             "graph pinned to [N, K] weights: nvteGemmF16 computes the tanh form only)")
         self.lm_head = lm_head
         if lm_head:
             assert self.drv.homBertEnableLmHead(self.h) == 0, "homBertEnableLmHead failed"

@@ -138,13 +138,19 @@ void gemm(HomBertEncoder *e, const Tensor &a, const Tensor &w, const Tensor &c,
 // layout: 0 row-major weight, 1 [N, K] weight, -1 decide here (gemmMode 0: always
 // [N, K]; 1: what the shipped table prefers; 2: what the live autotuner finds).
 // nvteGemmF16 computes the tanh form of GELU only, so a GELU role of an erf
-// graph stays on the manifest path.
-void chooseGemm(HomBertEncoder *e, int64_t M, int64_t N, int64_t K, int64_t act,
+// graph stays on the manifest path; pinning such a role to [N, K] is refused
+// (returns false) instead of silently computing the other GELU.
+bool chooseGemm(HomBertEncoder *e, int64_t M, int64_t N, int64_t K, int64_t act,
                 float beta, int layout, GemmChoice *out) {
   const bool nkAllowed = act == 0 || e->geluForm == 1 || e->gemmMode == 0;
   int64_t idx = -1;
   int32_t sk = 1;
   out->nk = false;
+  if (layout == 1 && !nkAllowed) {
+    fprintf(stderr, "hom_bert_driver: a GELU role of an erf-GELU graph cannot "
+                    "take [N, K] weights: nvteGemmF16 computes the tanh form\n");
+    return false;
+  }
   if (e->gemmMode == 0 || layout == 1) {
     out->nk = true;
   } else if (e->gemmMode == 2) {
@@ -161,6 +167,7 @@ void chooseGemm(HomBertEncoder *e, int64_t M, int64_t N, int64_t K, int64_t act,
   }
   out->gemmNum = out->nk ? 0 : int32_t(idx + 1);
   out->splitK = out->nk ? 1 : sk;
+  return true;
 }
 
 void callList(HomBertEncoder *e, int fromIds) {
@@ -225,10 +232,21 @@ homBertCreateWithLayout(int layers, int hidden, int heads, int ffn, int batch,
   {
     const int64_t M = int64_t(batch) * seq;
     const int64_t gelu = geluForm == 1 ? 2 : 1;
-    chooseGemm(e, M, 3 * hidden, hidden, 0, 0.0f, e->roleLayout[0], &e->cQkv);
-    chooseGemm(e, M, hidden, hidden, 0, 1.0f, e->roleLayout[1], &e->cOut);
-    chooseGemm(e, M, ffn, hidden, gelu, 0.0f, e->roleLayout[2], &e->cFfn1);
-    chooseGemm(e, M, hidden, ffn, 0, 1.0f, e->roleLayout[3], &e->cFfn2);
+    // the LM transform is a GELU role too; its layout is checked here so that
+    // a bad pin fails at creation, not at homBertEnableLmHead
+    const bool transformOk =
+        !(e->roleLayout[4] == 1 && geluForm == 0 && gemmMode != 0);
+    if (!chooseGemm(e, M, 3 * hidden, hidden, 0, 0.0f, e->roleLayout[0], &e->cQkv) ||
+        !chooseGemm(e, M, hidden, hidden, 0, 1.0f, e->roleLayout[1], &e->cOut) ||
+        !chooseGemm(e, M, ffn, hidden, gelu, 0.0f, e->roleLayout[2], &e->cFfn1) ||
+        !chooseGemm(e, M, hidden, ffn, 0, 1.0f, e->roleLayout[3], &e->cFfn2) ||
+        !transformOk) {
+      if (!transformOk)
+        fprintf(stderr, "hom_bert_driver: the LM transform of an erf-GELU graph "
+                        "cannot take [N, K] weights\n");
+      delete e;
+      return nullptr;
+    }
   }
   for (auto &w : e->w) {
     w.wqkv.m = e->cQkv.nk ? alloc3DMemRefNVGPUF16(1, 3 * hidden, hidden)
@@ -281,10 +299,11 @@ DRV_EXPORT int homBertEnableLmHead(HomBertEncoder *e) {
     return 0;
   {
     const int64_t M = int64_t(e->batch) * e->seq;
-    chooseGemm(e, M, e->hidden, e->hidden, e->geluForm == 1 ? 2 : 1, 0.0f,
-               e->roleLayout[4], &e->cTransform);
-    chooseGemm(e, M, e->vocab, e->hidden, 0, 0.0f, e->roleLayout[5],
-               &e->cDecoder);
+    if (!chooseGemm(e, M, e->hidden, e->hidden, e->geluForm == 1 ? 2 : 1, 0.0f,
+                    e->roleLayout[4], &e->cTransform) ||
+        !chooseGemm(e, M, e->vocab, e->hidden, 0, 0.0f, e->roleLayout[5],
+                    &e->cDecoder))
+      return -1;
   }
   e->wTransform.m = alloc3DMemRefNVGPUF16(1, e->hidden, e->hidden);
   e->wDecoder.m = e->cDecoder.nk
@@ -702,36 +721,76 @@ DRV_EXPORT double homTimeGemmNvte(int64_t M, int64_t N, int64_t K, int64_t act,
 }
 
 // In-place layer norm (reference form) when fused == 0; residual add + affine
-// layer norm (homAddLayernormF16) when fused != 0.
-DRV_EXPORT double homTimeLayernorm(int64_t rows, int64_t hidden, int fused,
-                                   int iters, int warmup) {
-  Tensor x, r, g, bt, o;
-  x.m = alloc3DMemRefNVGPUF16(1, int32_t(rows), int32_t(hidden));
-  r.m = alloc3DMemRefNVGPUF16(1, int32_t(rows), int32_t(hidden));
-  o.m = alloc3DMemRefNVGPUF16(1, int32_t(rows), int32_t(hidden));
+// layer norm (homAddLayernormF16) when fused != 0.  The calls walk round-robin
+// over `sets` independent sets of tensors (x; x, residual and output when
+// fused).  With one set the tensors stay in the 256 MB last-level cache from
+// launch to launch whenever they fit, and the figure is a cache rate; with
+// sets whose total size is several times that cache every launch reads from
+// and writes to HBM.
+DRV_EXPORT double homTimeLayernormRotating(int64_t rows, int64_t hidden,
+                                           int fused, int sets, int iters,
+                                           int warmup) {
+  if (sets < 1)
+    sets = 1;
+  const size_t nSets = size_t(sets), nFused = fused ? nSets : 0;
+  std::vector<Tensor> x(nSets), r(nFused), o(nFused);
+  Tensor g, bt;
   g.m = alloc3DMemRefNVGPUF16(1, 1, int32_t(hidden));
   bt.m = alloc3DMemRefNVGPUF16(1, 1, int32_t(hidden));
-  fillRandomF16(x.data(), rows * hidden, 1.0f, 4);
-  fillRandomF16(r.data(), rows * hidden, 1.0f, 5);
   fillRandomF16(g.data(), hidden, 0.02f, 6);
   fillRandomF16(bt.data(), hidden, 0.02f, 7);
-  double ms;
-  {
+  const size_t bytes = size_t(rows) * size_t(hidden) * 2;
+  bool ok = g.data() && bt.data();
+  for (int i = 0; i < sets && ok; i++) {
+    x[size_t(i)].m = alloc3DMemRefNVGPUF16(1, int32_t(rows), int32_t(hidden));
+    ok = x[size_t(i)].data() != nullptr;
+    if (fused && ok) {
+      r[size_t(i)].m = alloc3DMemRefNVGPUF16(1, int32_t(rows), int32_t(hidden));
+      o[size_t(i)].m = alloc3DMemRefNVGPUF16(1, int32_t(rows), int32_t(hidden));
+      ok = r[size_t(i)].data() && o[size_t(i)].data();
+    }
+    if (!ok)
+      break;
+    if (i == 0) {
+      fillRandomF16(x[0].data(), rows * hidden, 1.0f, 4);
+      if (fused)
+        fillRandomF16(r[0].data(), rows * hidden, 1.0f, 5);
+    } else {
+      (void)hipMemcpy(x[size_t(i)].data(), x[0].data(), bytes,
+                      hipMemcpyDeviceToDevice);
+      if (fused)
+        (void)hipMemcpy(r[size_t(i)].data(), r[0].data(), bytes,
+                        hipMemcpyDeviceToDevice);
+    }
+  }
+  double ms = -1.0;
+  if (ok) {
     Timer t;
+    int next = 0;
     ms = t.run(
         [&] {
+          const size_t i = size_t(next);
+          next = next + 1 == sets ? 0 : next + 1;
           if (fused)
-            homAddLayernormF16(3, x.m.descriptor, 3, r.m.descriptor, 3,
+            homAddLayernormF16(3, x[i].m.descriptor, 3, r[i].m.descriptor, 3,
                                g.m.descriptor, 3, bt.m.descriptor, 3,
-                               o.m.descriptor, 1e-12f);
+                               o[i].m.descriptor, 1e-12f);
           else
-            nvteLayernormF16(3, x.m.descriptor, 1e-12f);
+            nvteLayernormF16(3, x[i].m.descriptor, 1e-12f);
         },
         iters, warmup);
   }
-  for (Tensor *t : {&x, &r, &g, &bt, &o})
-    t->release();
+  for (auto *v : {&x, &r, &o})
+    for (Tensor &t : *v)
+      t.release();
+  g.release();
+  bt.release();
   return ms;
+}
+
+DRV_EXPORT double homTimeLayernorm(int64_t rows, int64_t hidden, int fused,
+                                   int iters, int warmup) {
+  return homTimeLayernormRotating(rows, hidden, fused, 1, iters, warmup);
 }
 
 // Packed-QKV attention with per-sequence valid lengths `lens` (host, int32[bs]).
@@ -764,26 +823,53 @@ DRV_EXPORT double homTimeAttention(int64_t bs, int64_t seq, int64_t heads,
   return ms;
 }
 
-DRV_EXPORT double homTimeElementwiseAdd(int64_t rows, int64_t hidden, int iters,
-                                        int warmup) {
-  Tensor a, b, o;
-  a.m = alloc3DMemRefNVGPUF16(1, int32_t(rows), int32_t(hidden));
-  b.m = alloc3DMemRefNVGPUF16(1, int32_t(rows), int32_t(hidden));
-  o.m = alloc3DMemRefNVGPUF16(1, int32_t(rows), int32_t(hidden));
-  fillRandomF16(a.data(), rows * hidden, 1.0f, 9);
-  fillRandomF16(b.data(), rows * hidden, 1.0f, 10);
-  double ms;
-  {
+// out = a + b over `sets` independent (a, b, out) triples walked round-robin
+// (see homTimeLayernormRotating for what the number of sets decides).
+DRV_EXPORT double homTimeElementwiseAddRotating(int64_t rows, int64_t hidden,
+                                                int sets, int iters,
+                                                int warmup) {
+  if (sets < 1)
+    sets = 1;
+  const size_t nSets = size_t(sets);
+  std::vector<Tensor> a(nSets), b(nSets), o(nSets);
+  const size_t bytes = size_t(rows) * size_t(hidden) * 2;
+  bool ok = true;
+  for (int i = 0; i < sets && ok; i++) {
+    const size_t k = size_t(i);
+    a[k].m = alloc3DMemRefNVGPUF16(1, int32_t(rows), int32_t(hidden));
+    b[k].m = alloc3DMemRefNVGPUF16(1, int32_t(rows), int32_t(hidden));
+    o[k].m = alloc3DMemRefNVGPUF16(1, int32_t(rows), int32_t(hidden));
+    ok = a[k].data() && b[k].data() && o[k].data();
+    if (!ok)
+      break;
+    if (i == 0) {
+      fillRandomF16(a[0].data(), rows * hidden, 1.0f, 9);
+      fillRandomF16(b[0].data(), rows * hidden, 1.0f, 10);
+    } else {
+      (void)hipMemcpy(a[k].data(), a[0].data(), bytes, hipMemcpyDeviceToDevice);
+      (void)hipMemcpy(b[k].data(), b[0].data(), bytes, hipMemcpyDeviceToDevice);
+    }
+  }
+  double ms = -1.0;
+  if (ok) {
     Timer t;
+    int next = 0;
     ms = t.run(
         [&] {
-          thrustElementwiseAddF16(3, a.m.descriptor, 3, b.m.descriptor, 3,
-                                  o.m.descriptor);
+          const size_t i = size_t(next);
+          next = next + 1 == sets ? 0 : next + 1;
+          thrustElementwiseAddF16(3, a[i].m.descriptor, 3, b[i].m.descriptor, 3,
+                                  o[i].m.descriptor);
         },
         iters, warmup);
   }
-  a.release();
-  b.release();
-  o.release();
+  for (auto *v : {&a, &b, &o})
+    for (Tensor &t : *v)
+      t.release();
   return ms;
+}
+
+DRV_EXPORT double homTimeElementwiseAdd(int64_t rows, int64_t hidden, int iters,
+                                        int warmup) {
+  return homTimeElementwiseAddRotating(rows, hidden, 1, iters, warmup);
 }

@@ -271,6 +271,18 @@ int32_t homGemmSelect(int64_t M, int64_t N, int64_t K, int64_t activation,
   return tuned ? 1 : 0;
 }
 
+int32_t homGemmSelectNvte(int64_t M, int64_t N, int64_t K, int64_t activation,
+                          int64_t *idx, int32_t *splitK) {
+  int64_t i = -1;
+  int32_t s = 1;
+  const bool tuned = selectGemmNvte(M, N, K, activation, &i, &s);
+  if (idx)
+    *idx = i;
+  if (splitK)
+    *splitK = s;
+  return tuned ? 1 : 0;
+}
+
 int32_t homGemmPrefersNvte(int64_t M, int64_t N, int64_t K, int64_t activation) {
   return gemmPrefersNvte(M, N, K, activation) ? 1 : 0;
 }

@@ -344,8 +344,26 @@ Status runGemmManifest(int64_t rankA, void *dstA, int64_t rankB, void *dstB,
       idx = fallbackKernel(gemmKernelInfo(idx).epilogue, cls);
       pr.splitK = 1;
     }
+    if (noAlloc) {
+      // The caller did not ask for split-K: a factor the library chose itself
+      // shrinks until its partial tiles fit the fixed array (1 needs none).
+      // An explicit gemmNum / splitK that does not fit is rejected by the launch.
+      const GemmKernelInfo &ki = gemmKernelInfo(idx);
+      const size_t perSlice = size_t((pr.M + ki.tileM - 1) / ki.tileM) *
+                              size_t((pr.N + ki.tileN - 1) / ki.tileN) *
+                              size_t(ki.tileM) * ki.tileN * sizeof(float);
+      while (pr.splitK > 1 && perSlice * size_t(pr.splitK) > pr.workspaceBytes)
+        pr.splitK--;
+    }
   }
   return launchGemm(idx, pr, stream());
+}
+
+bool selectGemmNvte(int64_t M, int64_t N, int64_t K, int64_t activation,
+                    int64_t *idx, int32_t *splitK) {
+  const Epilogue epi = epilogueFor(activation, true);
+  return selectGemm(M, N, K, epi == Epilogue::kGeluTanh ? 2 : activation, idx,
+                    splitK, true);
 }
 
 namespace {
@@ -353,8 +371,7 @@ int chooseNvteKernel(GemmProblem *pr, int64_t activation) {
   int64_t sel;
   int32_t sk;
   const Epilogue epi = epilogueFor(activation, true);
-  selectGemm(pr->M, pr->N, pr->K, epi == Epilogue::kGeluTanh ? 2 : activation,
-             &sel, &sk, true);
+  selectGemmNvte(pr->M, pr->N, pr->K, activation, &sel, &sk);
   int idx = int(sel);
   pr->splitK = sk;
   // Profiling knob: HOM_NVTE_GEMM_KERNEL="<manifest name>[,<splitK>]" pins the

@@ -39,6 +39,10 @@ Status runLayernormGemm(int64_t rankA, void *dstA, int64_t rankB, void *dstB,
 // shape was found in the tuned table.
 bool selectGemm(int64_t M, int64_t N, int64_t K, int64_t activation,
                 int64_t *idx, int32_t *splitK, bool bIsNK = false);
+// What nvteGemmF16 runs for a shape (B as [N, K]; activation 1 is the tanh
+// form there), before the per-call alignment fallback.
+bool selectGemmNvte(int64_t M, int64_t N, int64_t K, int64_t activation,
+                    int64_t *idx, int32_t *splitK);
 // Whether the tuned table says that, for this shape, the [N, K] path of
 // nvteGemmF16 beats every manifest kernel on row-major B (what the reference's
 // profiler reports as index -1).

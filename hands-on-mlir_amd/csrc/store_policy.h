@@ -31,7 +31,12 @@ __device__ __forceinline__ void storeWriteThrough(V *p, const V &v) {
                 "store width");
   if constexpr (sizeof(V) == 16) {
     typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-    asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1"
+    // The hardware needs two wait states between a store wider than 64
+    // bits and a vector instruction that overwrites its data registers.  The
+    // compiler inserts them for stores it emits itself but cannot see inside
+    // an asm statement, and the registers are dead right after it, so the
+    // wait states are part of the statement.
+    asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1\n\ts_nop 1"
                  :
                  : "v"(p), "v"(__builtin_bit_cast(u32x4, v))
                  : "memory");

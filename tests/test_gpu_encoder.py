@@ -45,22 +45,39 @@ def lm_head_oracle(oracle, h16, model, gelu, rows=None):
     return oracle.gemm(t, model["word"], b_is_nk=True)
 
 
-def check(got, want32, lens, what, rel_limit=1e-3, outlier_frac=0.0):
-    """Elementwise |got - want| <= 1e-2 + 1e-3 |want| on the valid positions plus a norm-wise bound.
-    outlier_frac > 0 (only for comparisons of an fp16-storage pipeline with the fp32 reference over a
-    whole 12-layer stack, where the error is accumulated rounding noise with a tail): that fraction of a
-    sequence's elements may lie outside the elementwise bound, none outside twice the bound."""
-    errs, norms = 0.0, 0.0
+def outliers(got, want32, lens, atol=1e-2, rtol=1e-3):
+    """Elements of the valid positions outside atol + rtol |want|: (count, worst error, its bound, its index)."""
+    count, worst = 0, (0.0, 0.0, None)
     for b, n in enumerate(lens):
         g, w = got[b, :n].astype(np.float64), want32[b, :n].astype(np.float64)
         err = np.abs(g - w)
-        bound = 1e-2 + 1e-3 * np.abs(w)
-        bad = err > bound
-        assert bad.sum() <= np.ceil(outlier_frac * bad.size) and not (err > 2 * bound).any(), \
-            f"{what}: batch {b}: {bad.sum()} of {bad.size} elements off, max {err.max():.3e}"
-        errs += (err ** 2).sum()
+        bound = atol + rtol * np.abs(w)
+        count += int((err > bound).sum())
+        i = np.unravel_index(np.argmax(err - bound), err.shape)
+        if worst[2] is None or err[i] - bound[i] > worst[0] - worst[1]:
+            worst = (float(err[i]), float(bound[i]), (b,) + tuple(int(v) for v in i))
+    return count, worst
+
+
+def relerr(got, want32, lens):
+    errs, norms = 0.0, 0.0
+    for b, n in enumerate(lens):
+        g, w = got[b, :n].astype(np.float64), want32[b, :n].astype(np.float64)
+        errs += ((g - w) ** 2).sum()
         norms += (w ** 2).sum()
-    rel = np.sqrt(errs / norms)
+    return np.sqrt(errs / norms)
+
+
+def check(got, want32, lens, what, rel_limit=1e-3, allowed_outliers=0):
+    """Elementwise |got - want| <= 1e-2 + 1e-3 |want| on the valid positions plus a norm-wise bound.
+    allowed_outliers is never a constant: a caller that compares an fp16-storage pipeline with the fp32
+    reference over a whole layer stack passes what the oracle's own fp16 pipeline shows against the same
+    reference (+ 1), so the GPU path may have the noise tail fp16 storage has and nothing more."""
+    count, (err, bound, where) = outliers(got, want32, lens)
+    assert count <= allowed_outliers, \
+        f"{what}: {count} elements off (allowed {allowed_outliers}), worst {err:.3e} against {bound:.3e} at {where}"
+    assert err <= 2 * bound, f"{what}: element {where} is {err:.3e} off, more than twice its bound {bound:.3e}"
+    rel = relerr(got, want32, lens)
     assert rel <= rel_limit, f"{what}: norm-wise relative error {rel:.3e} > {rel_limit}"
     return rel
 
@@ -186,6 +203,22 @@ def test_mixed_weight_layouts_per_role(gpu, oracle, synth):
                     enc.set_gemm_choice("out", 1, 1)
         finally:
             enc.close()
+    # an erf-GELU graph: the linear roles may still go to nvteGemmF16, and the result is the erf encoder
+    want_erf = oracle_forward(oracle, model, "erf")
+    enc = bert.BertEncoder(2, 128, 2, 512, 3, 64, 1000, gemm_mode=1, gelu_form="erf",
+                           role_layout={"qkv": "nk", "out": "nk", "ffn2": "nk"})
+    try:
+        assert not enc.role_is_nk("ffn1")
+        enc.load(model)
+        enc.set_inputs(ids=model["ids"], mask=model["mask"])
+        enc.forward()
+        check(enc.output(), want_erf, model["lens"], "erf graph with [N, K] linear roles")
+    finally:
+        enc.close()
+    # nvteGemmF16 computes the tanh form only: pinning a GELU role of an erf graph to it is refused
+    for lay in ({"ffn1": "nk"}, {"transform": "nk"}):
+        with pytest.raises(ValueError):
+            bert.BertEncoder(2, 128, 2, 512, 3, 64, 1000, gemm_mode=1, gelu_form="erf", role_layout=lay)
 
 
 def test_pinned_gemm_kernels_in_the_graph(gpu, rt, oracle, synth):
@@ -277,10 +310,17 @@ def test_bert_base_b8_s128(gpu, oracle, synth):
         # (2) against the fp32 reference of the same weights and inputs (no intermediate
         # rounding): the GPU path must be as close to it as the fp16-faithful oracle is,
         # i.e. fp16 storage -- which the boundary fixes -- is the only error source.
+        # Elementwise, the same rule: the GPU path may have as many elements outside rtol 1e-3 /
+        # atol 1e-2 as the oracle's own fp16 pipeline has against the fp32 reference, plus one.
         pure = oracle_forward(oracle, model, "erf", round_intermediates=False)
-        rel32 = check(got, pure, model["lens"], "BERT-base vs fp32 reference", rel_limit=2e-3, outlier_frac=1e-5)
-        floor = check(faithful.astype(np.float16), pure, model["lens"], "fp16-faithful oracle vs fp32 reference",
-                      rel_limit=2e-3, outlier_frac=1e-5)
+        floor_out, floor_worst = outliers(faithful.astype(np.float16), pure, model["lens"])
+        gpu_out, gpu_worst = outliers(got, pure, model["lens"])
+        print(f"BERT-base e2e elements outside rtol 1e-3 / atol 1e-2 of the fp32 reference: GPU {gpu_out} "
+              f"(worst {gpu_worst[0]:.3e} against {gpu_worst[1]:.3e} at {gpu_worst[2]}), oracle's fp16 pipeline "
+              f"{floor_out} (worst {floor_worst[0]:.3e} against {floor_worst[1]:.3e} at {floor_worst[2]})")
+        floor = relerr(faithful.astype(np.float16), pure, model["lens"])
+        rel32 = check(got, pure, model["lens"], "BERT-base vs fp32 reference", rel_limit=2e-3,
+                      allowed_outliers=floor_out + 1)
         print(f"BERT-base e2e norm-wise relative error: {rel16:.3e} vs fp16-faithful oracle, "
               f"{rel32:.3e} vs fp32 reference (fp16-storage floor {floor:.3e})")
         assert rel32 <= 1.1 * floor, f"GPU path error {rel32:.3e} exceeds the fp16-storage floor {floor:.3e}"
@@ -320,14 +360,14 @@ def test_single_layer_full_width(gpu, oracle, synth):
             enc.close()
 
 
-def ref_flags(got, want32, lens):
+def ref_flags(got, want32, lens, thr=1e-2):
     """The reference driver's own criterion (examples/torch/bert/bert.cu:148-153): an
-    element is wrong only when both its absolute and its relative error exceed 1e-2."""
+    element is wrong only when both its absolute and its relative error exceed 1e-2 (thr)."""
     bad = 0
     for b, n in enumerate(lens):
         g, w = got[b, :n].astype(np.float64), want32[b, :n].astype(np.float64)
         err = np.abs(g - w)
-        bad += int(((err > 1e-2) & (err > 1e-2 * np.abs(w))).sum())
+        bad += int(((err > thr) & (err > thr * np.abs(w))).sum())
     return bad
 
 
@@ -357,27 +397,25 @@ def test_bert_large_architecture(gpu, oracle, synth):
     faithful = oracle_forward(oracle, small, "erf")
     pure = oracle_forward(oracle, small, "erf", round_intermediates=False)
 
-    def relerr(a, b):
-        e = n = 0.0
-        for s, ln in enumerate(small["lens"]):
-            x, y = a[s, :ln].astype(np.float64), b[s, :ln].astype(np.float64)
-            e += ((x - y) ** 2).sum()
-            n += (y ** 2).sum()
-        return np.sqrt(e / n)
-
-    rel16, rel32 = relerr(got2, faithful), relerr(got2, pure)
-    floor = relerr(faithful.astype(np.float16), pure)
+    lens2 = small["lens"]
+    rel16, rel32 = relerr(got2, faithful, lens2), relerr(got2, pure, lens2)
+    floor = relerr(faithful.astype(np.float16), pure, lens2)
     print(f"BERT-large b2 s512 norm-wise relative error: {rel16:.3e} vs fp16-faithful oracle, "
           f"{rel32:.3e} vs fp32 reference (fp16-storage floor {floor:.3e})")
     # The rounding noise of 24 layers of fp16 storage (rms 1.5e-3 on unit-variance
     # outputs, the same for the oracle's own fp16 pipeline) puts the reference's 1e-2
-    # threshold at ~7 sigma: allow its tail, 1e-5 of the elements.
+    # threshold at ~7 sigma, so a few elements of its tail show.  The allowance is what the
+    # oracle's own fp16 pipeline shows against the fp32 reference, plus one; against the
+    # fp16-faithful oracle (two noisy pipelines) it follows from the triangle inequality:
+    # an element 1e-2 apart there is at least 5e-3 from the fp32 reference in one of the two.
     valid = int(sum(small["lens"])) * 1024
     flags16, flags32 = ref_flags(got2, faithful, small["lens"]), ref_flags(got2, pure, small["lens"])
     flags_floor = ref_flags(faithful.astype(np.float16), pure, small["lens"])
-    print(f"elements beyond the reference's criterion: {flags16} vs fp16-faithful oracle, {flags32} vs fp32 "
-          f"reference, {flags_floor} for the oracle's own fp16 pipeline vs fp32 (of {valid})")
-    assert flags16 <= 1e-5 * valid and flags32 <= 1e-5 * valid
+    half = (ref_flags(got2, pure, small["lens"], 5e-3) +
+            ref_flags(faithful.astype(np.float16), pure, small["lens"], 5e-3))
+    print(f"elements beyond the reference's criterion: {flags16} vs fp16-faithful oracle (bound {half}), {flags32} "
+          f"vs fp32 reference, {flags_floor} for the oracle's own fp16 pipeline vs fp32 (of {valid})")
+    assert flags32 <= flags_floor + 1 and flags16 <= half
     # 24 layers of decorrelating fp16 rounding noise: sqrt(2) x the 12-layer bound
     assert rel16 <= 3e-3 and rel32 <= 3e-3
     assert rel32 <= 1.1 * floor, f"GPU path error {rel32:.3e} exceeds the fp16-storage floor {floor:.3e}"
@@ -392,8 +430,8 @@ def test_bert_large_architecture(gpu, oracle, synth):
         assert np.isfinite(got32.astype(np.float32)).all()
         # same sequences inside the full batch: other tiles and split-K choices, so equal
         # up to the fp16 rounding noise measured above, not bit for bit
-        assert ref_flags(got32[:2], got2.astype(np.float32), small["lens"]) <= 1e-5 * valid
-        drift = relerr(got32[:2], got2.astype(np.float32))
+        assert ref_flags(got32[:2], pure, small["lens"]) <= flags_floor + 1
+        drift = relerr(got32[:2], got2.astype(np.float32), lens2)
         print(f"BERT-large b32 vs b2 on the shared sequences: norm-wise {drift:.3e}")
         assert drift <= 3e-3
         # padding content and neighbours do not matter (same launch shapes: bit exact)

@@ -120,7 +120,16 @@ def test_row_stats_constant_row_is_finite(oracle):
     x[2] = 1000.25
     var, mean = oracle.row_stats(x, 1e-12)
     assert np.isfinite(var).all() and np.isfinite(mean).all()
-    assert np.allclose(var, 1e6, rtol=1e-3) or (var > 1e3).all()
+    # The true variance of a constant row is exactly 0, so var = 1/sqrt(eps) = 1e6 wherever the fp64
+    # rounding of E[x^2] - E[x]^2 (at most 2 n 2^-53 x^2, a sequential sum of n products) is far below
+    # eps, and never above it (the clamp); where the rounding is comparable to eps it can only lower var,
+    # to no less than 1/sqrt(that bound + eps).  mean is -x * var in every case.
+    xs = x[:, 0].astype(np.float64)
+    slack = 2 * 768 * 2.0 ** -53 * xs ** 2
+    assert (var <= 1e6 * (1 + 1e-6)).all()
+    assert (var >= (1 - 1e-6) / np.sqrt(slack + 1e-12)).all()
+    assert slack[0] < 1e-14 and abs(var[0] - 1e6) <= 1e-3 * 1e6
+    assert np.allclose(mean, -xs * var.astype(np.float64), rtol=1e-6, atol=0)
     # a row with spread is untouched by the clamp
     g = np.random.default_rng(5)
     y = g.standard_normal((4, 64)).astype(np.float32)

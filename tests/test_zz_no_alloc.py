@@ -51,7 +51,9 @@ def test_no_alloc_gemm_matches_allocating_entry_point(gpu, rt, oracle):
         C = g.standard_normal((1, M_, N_)).astype(np.float16) if with_c else None
         beta = 1.0 if with_c else 0.0
         want = _run(gpu.cutlassGemmF16, rt, A, B, C, beta, num, sk)
+        generation = gpu.homScratchGeneration()
         got = _run(gpu.homGemmF16NoAlloc, rt, A, B, C, beta, num, sk)
+        assert gpu.homScratchGeneration() == generation, "the no-alloc entry point grew the library's scratch"
         assert np.array_equal(got, want), f"no-alloc GEMM differs from cutlassGemmF16 at {(M_, N_, K_, sk)}"
         ref = oracle.gemm(A[0], B[0], C[0] if with_c else None, beta=beta)
         err = np.abs(got[0].astype(np.float64) - ref)
@@ -61,6 +63,22 @@ def test_no_alloc_gemm_matches_allocating_entry_point(gpu, rt, oracle):
     B = (g.standard_normal((1, 4096, 1024)) * 0.02).astype(np.float16)
     assert np.array_equal(_run(gpu.homGemmF16NoAlloc, rt, A, B, None, 0.0, 0, 1),
                           _run(gpu.cutlassGemmF16, rt, A, B, None, 0.0, 0, 1))
+
+
+def test_no_alloc_gemm_shrinks_a_split_k_it_chose_itself(gpu, rt, oracle):
+    """gemmNum 0 leaves kernel and split-K to the library.  Whatever it picks, the call must neither
+    allocate nor fail for a problem whose sliced partial tiles could exceed the array: 4096 x 4096
+    outputs are 64 MiB per slice, so any factor above 1 is shrunk to 1."""
+    g = np.random.default_rng(78)
+    A = g.standard_normal((1, 4096, 256)).astype(np.float16)
+    B = (g.standard_normal((1, 256, 4096)) * 0.05).astype(np.float16)
+    generation = gpu.homScratchGeneration()
+    got = _run(gpu.homGemmF16NoAlloc, rt, A, B, None, 0.0, 0, 1)
+    assert gpu.homScratchGeneration() == generation
+    rows = np.arange(0, 4096, 97)
+    ref = oracle.gemm(np.ascontiguousarray(A[0][rows]), B[0])
+    err = np.abs(got[0][rows].astype(np.float64) - ref)
+    assert (err <= GEMM_TOL["atol"] + GEMM_TOL["rtol"] * np.abs(ref)).all(), err.max()
 
 
 def test_no_alloc_gemm_rejects_oversized_split_k(gpu, rt):
