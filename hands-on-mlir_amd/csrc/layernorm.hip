@@ -29,105 +29,16 @@ template <> struct Vec16<float> {
   typedef float type __attribute__((ext_vector_type(4)));
 };
 
-// One wavefront per row; VPL 16-byte vectors per lane.  The streaming form,
-// for tensors beyond the last-level cache: bandwidth bound, default stores.
-template <typename T, int VPL, bool HAS_RES, bool HAS_AFFINE>
-__global__ __launch_bounds__(256) void layernormStreamKernel(
-    const T *x, const T *res,
-    const T *__restrict__ gamma, const T *__restrict__ beta, T *out,
-    int64_t rows, int hidden, float eps) {
-  using V = typename Vec16<T>::type;
-  constexpr int N = Vec16<T>::kN;
-  const int lane = threadIdx.x & (kWave - 1);
-  const int64_t row = int64_t(blockIdx.x) * (blockDim.x / kWave) +
-                      (threadIdx.x / kWave);
-  if (row >= rows)
-    return;
-  const int nvec = hidden / N;
-  const V *xr = reinterpret_cast<const V *>(x + row * hidden);
-  const V *rr = HAS_RES ? reinterpret_cast<const V *>(res + row * hidden)
-                        : nullptr;
-
-  float v[VPL][N];
-  V raw[VPL];
-  V rawRes[VPL];
-#pragma unroll
-  for (int i = 0; i < VPL; i++) {
-    const int idx = lane + i * kWave;
-    if (idx < nvec) {
-      raw[i] = xr[idx];
-      if (HAS_RES)
-        rawRes[i] = rr[idx];
-    }
-  }
-  float sum = 0.f;
-#pragma unroll
-  for (int i = 0; i < VPL; i++) {
-    const int idx = lane + i * kWave;
-#pragma unroll
-    for (int j = 0; j < N; j++) {
-      float f = 0.f;
-      if (idx < nvec) {
-        f = float(raw[i][j]);
-        if (HAS_RES)
-          f += float(rawRes[i][j]); // the sum stays in fp32
-      }
-      v[i][j] = f;
-      sum += f;
-    }
-  }
-  const float invH = 1.0f / float(hidden);
-  const float mean = waveSum(sum) * invH;
-  float sq = 0.f;
-#pragma unroll
-  for (int i = 0; i < VPL; i++) {
-    const int idx = lane + i * kWave;
-    if (idx < nvec) {
-#pragma unroll
-      for (int j = 0; j < N; j++) {
-        const float d = v[i][j] - mean;
-        sq += d * d;
-      }
-    }
-  }
-  const float var = waveSum(sq) * invH;
-  const float rstd = 1.0f / sqrtf(var + eps);
-
-  V *orow = reinterpret_cast<V *>(out + row * hidden);
-#pragma unroll
-  for (int i = 0; i < VPL; i++) {
-    const int idx = lane + i * kWave;
-    if (idx < nvec) {
-      V o;
-      if (HAS_AFFINE) {
-        V g, b;
-        bool hasG = gamma != nullptr, hasB = beta != nullptr;
-        if (hasG)
-          g = reinterpret_cast<const V *>(gamma)[idx];
-        if (hasB)
-          b = reinterpret_cast<const V *>(beta)[idx];
-#pragma unroll
-        for (int j = 0; j < N; j++) {
-          float y = (v[i][j] - mean) * rstd;
-          if (hasG)
-            y *= float(g[j]);
-          if (hasB)
-            y += float(b[j]);
-          o[j] = T(y);
-        }
-      } else {
-#pragma unroll
-        for (int j = 0; j < N; j++)
-          o[j] = T((v[i][j] - mean) * rstd);
-      }
-      orow[idx] = o;
-    }
-  }
-}
-
-// One wavefront per row; VPL 16-byte vectors per lane.  The form for tensors of
-// a few megabytes, which the next kernel of the stream finds in the last-level
-// cache (results written through, see store_policy.h).
+// One wavefront per row; VPL 16-byte vectors per lane.
+//
+// STREAM == false: tensors of a few megabytes, which the next kernel of the
+// stream finds in the last-level cache (results written through, see
+// store_policy.h).  STREAM == true: tensors beyond that cache; rows are read
+// and written with the non-temporal hint, because nothing is touched twice and
+// without the hint the written rows linger in the L2s and compete with the
+// reads on their way out (16384 x 1024 in place, rotating over 800 MB so that
+// every launch is cold: 4.5 TB/s with default accesses, 5.4 TB/s with the hint;
+// a plain read-modify-write probe shows the same 4.7 -> 5.65 TB/s).
 //
 // The kernel is a chain of memory round trips (arguments, row, result) a few
 // hundred nanoseconds each, so everything it will read is requested at once and
@@ -135,7 +46,7 @@ __global__ __launch_bounds__(256) void layernormStreamKernel(
 // (768 columns: lanes 32..63 of the second vector) and a wavefront past the
 // last row load a valid address again and mask the values, instead of a branch
 // around the load, which would make the second request wait for the first.
-template <typename T, int VPL, bool HAS_RES, bool HAS_AFFINE>
+template <typename T, int VPL, bool HAS_RES, bool HAS_AFFINE, bool STREAM>
 __global__ __launch_bounds__(256) void layernormWaveKernel(
     const T *x, const T *res,
     const T *__restrict__ gamma, const T *__restrict__ beta, T *out,
@@ -163,9 +74,9 @@ __global__ __launch_bounds__(256) void layernormWaveKernel(
   for (int i = 0; i < VPL; i++) {
     const int idx = lane + i * kWave;
     const int at = idx < nvec ? idx : 0;
-    raw[i] = xr[at];
+    raw[i] = STREAM ? __builtin_nontemporal_load(&xr[at]) : xr[at];
     if (HAS_RES)
-      rawRes[i] = rr[at];
+      rawRes[i] = STREAM ? __builtin_nontemporal_load(&rr[at]) : rr[at];
     if (HAS_AFFINE) {
       // (null gamma / beta: wave-uniform branches, taken by nobody or everybody)
       if (hasG)
@@ -221,7 +132,10 @@ __global__ __launch_bounds__(256) void layernormWaveKernel(
       o[j] = T(y);
     }
     if (rowOk && idx < nvec) {
-      storeWriteThrough(&orow[idx], o);
+      if (STREAM)
+        __builtin_nontemporal_store(o, &orow[idx]);
+      else
+        storeWriteThrough(&orow[idx], o);
     }
   }
 }
@@ -281,26 +195,24 @@ __global__ __launch_bounds__(256) void layernormBlockKernel(
 }
 
 // Results that the next kernel of the stream will find in the last-level cache
-// (a few megabytes) take the latency-oriented kernel with write-through stores;
-// streaming-size tensors take the bandwidth-oriented one (16384 x 1024: 9.8 us
-// against 10.4 us with the other).
+// (a few megabytes) are written through; larger tensors stream.
 constexpr int64_t kSmallTensorBytes = int64_t(16) << 20;
 
-#define HOM_LN_LAUNCH(KERNEL)                                                  \
+#define HOM_LN_LAUNCH(KERNEL, ...)                                             \
   do {                                                                         \
     if (res) {                                                                 \
       if (affine)                                                              \
-        KERNEL<T, VPL, true, true>                                             \
+        KERNEL<T, VPL, true, true, ##__VA_ARGS__>                              \
             <<<grid, block, 0, s>>>(x, res, gamma, beta, out, rows, hidden, eps); \
       else                                                                     \
-        KERNEL<T, VPL, true, false>                                            \
+        KERNEL<T, VPL, true, false, ##__VA_ARGS__>                             \
             <<<grid, block, 0, s>>>(x, res, gamma, beta, out, rows, hidden, eps); \
     } else {                                                                   \
       if (affine)                                                              \
-        KERNEL<T, VPL, false, true>                                            \
+        KERNEL<T, VPL, false, true, ##__VA_ARGS__>                             \
             <<<grid, block, 0, s>>>(x, res, gamma, beta, out, rows, hidden, eps); \
       else                                                                     \
-        KERNEL<T, VPL, false, false>                                           \
+        KERNEL<T, VPL, false, false, ##__VA_ARGS__>                            \
             <<<grid, block, 0, s>>>(x, res, gamma, beta, out, rows, hidden, eps); \
     }                                                                          \
   } while (0)
@@ -311,10 +223,15 @@ void launchWave(const T *x, const T *res, const T *gamma, const T *beta, T *out,
   const int rowsPerBlock = 256 / kWave;
   dim3 grid((unsigned)((rows + rowsPerBlock - 1) / rowsPerBlock)), block(256);
   const bool affine = gamma || beta;
-  if (rows * hidden * int64_t(sizeof(T)) <= kSmallTensorBytes)
-    HOM_LN_LAUNCH(layernormWaveKernel);
-  else
-    HOM_LN_LAUNCH(layernormStreamKernel);
+  if (rows * hidden * int64_t(sizeof(T)) <= kSmallTensorBytes) {
+    HOM_LN_LAUNCH(layernormWaveKernel, false);
+  } else {
+    // (a persistent variant whose wavefronts keep their next row in flight
+    // while they reduce and store the current one measured the same 12.3-12.6
+    // us on 16384 x 1024 cold, at 2 to 8 workgroups per CU: the rate is the
+    // memory system's for a read-modify-write stream of this size)
+    HOM_LN_LAUNCH(layernormWaveKernel, true);
+  }
 }
 #undef HOM_LN_LAUNCH
 
