@@ -1,6 +1,9 @@
 """Tiny single-kernel workloads to run under rocprofv3 (kernel trace or --pmc).
 
-    python3 hands-on-mlir_amd/profile_kernels.py <what> [iters]
+    python3 hands-on-mlir_amd/profile_kernels.py <what> [iters] [tile]
+
+tile (GEMM workloads only): run the manifest kernel whose name holds `_<tile>_`
+(e.g. 256x256_64x2r1_w2x2) instead of the tuned one.
 
 what:  gemm1      FFN1 GEMM + bias + tanh-GELU, M=1024 K=768 N=3072 (tuned kernel)
        gemm5      BERT-large FFN2 GEMM, M=16384 K=4096 N=1024
@@ -30,16 +33,26 @@ def main():
     rt = importlib.import_module("hands-on-mlir_amd.hom_runtime")
     drv, lib = rt.load_driver(), rt.load_runtime()
     idx, sk = ctypes.c_int64(), ctypes.c_int32()
+    tile = sys.argv[3] if len(sys.argv) > 3 else None
+
+    def pick(m, n, k, act):
+        lib.homGemmSelect(m, n, k, act, ctypes.byref(idx), ctypes.byref(sk))
+        if tile:
+            want = {0: "_linear", 1: "_gelu", 2: "_gelutanh"}[act]
+            hits = [i for i, name, _, _ in rt.manifest() if f"_{tile}_" in name and name.endswith(want)]
+            assert hits, f"no manifest kernel matches {tile}"
+            idx.value, sk.value = hits[0], 1
+
     if what == "gemm1":
-        lib.homGemmSelect(1024, 3072, 768, 2, ctypes.byref(idx), ctypes.byref(sk))
+        pick(1024, 3072, 768, 2)
         ms = drv.homTimeGemm(1024, 3072, 768, 2, 1, idx.value + 1, sk.value, iters, 3)
         print(f"gemm1 {lib.homGemmManifestName(idx.value).decode()} splitK {sk.value}: {ms * 1e3:.2f} us")
     elif what == "gemm5":
-        lib.homGemmSelect(16384, 1024, 4096, 0, ctypes.byref(idx), ctypes.byref(sk))
+        pick(16384, 1024, 4096, 0)
         ms = drv.homTimeGemm(16384, 1024, 4096, 0, 0, idx.value + 1, sk.value, iters, 3)
         print(f"gemm5 {lib.homGemmManifestName(idx.value).decode()} splitK {sk.value}: {ms * 1e3:.2f} us")
     elif what == "gemm5g":
-        lib.homGemmSelect(16384, 4096, 1024, 1, ctypes.byref(idx), ctypes.byref(sk))
+        pick(16384, 4096, 1024, 1)
         ms = drv.homTimeGemm(16384, 4096, 1024, 1, 1, idx.value + 1, sk.value, iters, 3)
         print(f"gemm5g {lib.homGemmManifestName(idx.value).decode()} splitK {sk.value}: {ms * 1e3:.2f} us")
     elif what == "layernorm":

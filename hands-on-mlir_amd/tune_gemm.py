@@ -17,6 +17,10 @@ and over the two weight layouts, keeping a change only if the whole forward
 gets faster.
 
     HOM_PROFILE_BUDGET_MS=150 python hands-on-mlir_amd/tune_gemm.py [output.inc]     # needs a GPU
+
+--rows=16384[,...] retunes only the shapes with those row counts (and runs the
+in-graph pass only for the encoder with such a row count) and keeps the other
+rows of the existing table as they are.
 """
 import ctypes
 import importlib
@@ -41,8 +45,28 @@ def bert_shapes():
 # (BM, BN, WM, WN, slabs in flight, staging: "x2r" registers + 2 LDS buffers, "q" buffer_load ... lds into a ring)
 TILES = [(64, 64, 2, 2, 2, "x2r"), (64, 64, 2, 2, 4, "x2r"), (128, 64, 2, 2, 2, "x2r"), (64, 128, 2, 2, 2, "x2r"),
          (128, 128, 2, 4, 2, "x2r"), (128, 256, 2, 4, 2, "x2r"), (256, 128, 4, 2, 2, "x2r"), (256, 256, 2, 4, 1, "x2r"),
-         (128, 96, 4, 1, 2, "x2r"), (256, 96, 4, 1, 2, "x2r"),
-         (128, 128, 2, 4, 2, "q"), (128, 128, 2, 4, 3, "q"), (64, 64, 2, 2, 3, "q"), (256, 256, 2, 4, 1, "q")]
+         (256, 256, 2, 2, 1, "x2r"), (128, 96, 4, 1, 2, "x2r"), (256, 96, 4, 1, 2, "x2r"),
+         (128, 128, 2, 4, 2, "q"), (128, 128, 2, 4, 3, "q"), (64, 64, 2, 2, 3, "q"), (256, 256, 2, 4, 1, "q"),
+         # the 16x16x32-MFMA family (tile sides in steps of 16)
+         (128, 96, 4, 2, 2, "fine"), (64, 48, 4, 1, 2, "fine"), (64, 144, 4, 1, 2, "fine")]
+
+
+def tile_name(bm, bn, wm, wn, depth, staging, epi):
+    if staging == "fine":
+        return f"hom_gfx950_mfma_f16_s16x16x32gemm_f16_{bm}x{bn}_64x2r{depth}_w{wm}x{wn}_nn_align8_{epi}"
+    return f"hom_gfx950_mfma_f16_s32x32x16gemm_f16_{bm}x{bn}_64{staging}{depth}_w{wm}x{wn}_nn_align8_{epi}"
+
+
+def read_table(path):
+    """{(M, N, K, act): source line} of an existing table file."""
+    import re
+    rows = {}
+    if os.path.exists(path):
+        for line in open(path):
+            m = re.match(r"\s*\{(\d+), (\d+), (\d+), (\d+),", line)
+            if m:
+                rows[tuple(int(v) for v in m.groups())] = line.rstrip("\n")
+    return rows
 
 
 class Row:
@@ -64,13 +88,15 @@ class Row:
                 f'[N,K] {self.nk_us:.2f} us{self.note}')
 
 
-def in_graph_pass(rt, table):
+def in_graph_pass(rt, table, only_rows=None):
     """table: {(M, N, K, act): Row}; edited in place."""
     synth = importlib.import_module("hands-on-mlir_amd.synth")
     bert = importlib.import_module("hands-on-mlir_amd.bert")
     number = {n: i + 1 for i, n, _, _ in rt.manifest()}
     for kwargs, steps in [(dict(), 200),
                           (dict(layers=24, hidden=1024, heads=16, ffn=4096, bs=32, seq=512, config=41), 10)]:
+        if only_rows and kwargs.get("bs", 8) * kwargs.get("seq", 128) not in only_rows:
+            continue
         model = synth.bert_encoder(**kwargs)
         d = model["dims"]
         M, H, F = d["bs"] * d["seq"], d["hidden"], d["ffn"]
@@ -99,8 +125,7 @@ def in_graph_pass(rt, table):
                 best_us, best = forward_us(enc), None
                 epi = "gelu" if key[3] == 1 else "linear"
                 for (bm, bn, wm, wn, depth, staging) in TILES:
-                    name = (f"hom_gfx950_mfma_f16_s32x32x16gemm_f16_{bm}x{bn}_64{staging}{depth}_w{wm}x{wn}"
-                            f"_nn_align8_{epi}")
+                    name = tile_name(bm, bn, wm, wn, depth, staging, epi)
                     if number[name] == start[0]:
                         continue
                     enc.set_gemm_choice(role, number[name], 1)
@@ -140,7 +165,13 @@ def main():
     lib = rt.load_runtime()
     names = {i: n for i, n, _, _ in rt.manifest()}
     table = {}
+    only_rows = None
+    for a in sys.argv[1:]:
+        if a.startswith("--rows="):
+            only_rows = {int(v) for v in a[len("--rows="):].split(",")}
     for (M, N, K, act) in bert_shapes():
+        if only_rows and M not in only_rows:
+            continue
         beta = 1.0 if (act == 0 and N in (768, 1024) and K != N // 3) else 0.0
         res = []
         for nk in (0, 1):
@@ -153,9 +184,20 @@ def main():
         table[(M, N, K, act)] = Row(*res[0], *res[1])
         print(table[(M, N, K, act)].line((M, N, K, act)), flush=True)
     if "--no-in-graph" not in sys.argv:
-        in_graph_pass(rt, table)
+        in_graph_pass(rt, table, only_rows)
     args = [a for a in sys.argv[1:] if not a.startswith("--")]
     out = args[0] if args else os.path.join(HERE, "csrc", "gemm_tuned_table.inc")
+    if only_rows:
+        kept = read_table(os.path.join(HERE, "csrc", "gemm_tuned_table.inc"))
+        lines = [table[key].line(key) if key in table else line for key, line in kept.items()]
+        lines += [row.line(key) for key, row in table.items() if key not in kept]
+        with open(out, "w") as f:
+            f.write("// (M, N, K, activation: 0 linear / 1 GELU erf / 2 GELU tanh, kernel for row-major B, its split-K,\n"
+                    "//  kernel for B as [N, K] or nullptr, its split-K, 1 if the [N, K] path is the faster one)\n"
+                    "// Written by hands-on-mlir_amd/tune_gemm.py on an MI355X; do not edit by hand.\n")
+            f.write("\n".join(lines) + "\n")
+        print("wrote", out)
+        return
     with open(out, "w") as f:
         f.write("// (M, N, K, activation: 0 linear / 1 GELU erf / 2 GELU tanh, kernel for row-major B, its split-K,\n"
                 "//  kernel for B as [N, K] or nullptr, its split-K, 1 if the [N, K] path is the faster one)\n"
