@@ -242,7 +242,31 @@ def main():
         big_flops = 24 * (2.0 * 16384 * 1024 * (3 * 1024 + 1024 + 2 * 4096) + attn_flops)
         kernels["bert_large_b32_s512_encoder"] = {"ms": big_ms, "sequences/s": 32 / (big_ms * 1e-3),
                                                   "TFLOP/s": big_flops / (big_ms * 1e-3) / 1e12}
+        # the optional call list with the per-layer layer norms folded into the GEMMs around them
+        # (5 launches per layer instead of 7; not the reference's call list, reported beside it)
+        if args.gemm_mode != 0:
+            enc = bert.BertEncoder(24, 1024, 16, 4096, 32, 512, big["dims"]["vocab"],
+                                   gemm_mode=args.gemm_mode, gelu_form="erf", fold_layernorm=True)
+            enc.load(big)
+            enc.set_inputs(ids=big["ids"], mask=big["mask"])
+            fold_ms = enc.time(30, 15, graph=not args.eager)
+            enc.close()
+            kernels["bert_large_b32_s512_encoder_folded_layernorm"] = {
+                "ms": fold_ms, "sequences/s": 32 / (fold_ms * 1e-3), "TFLOP/s": big_flops / (fold_ms * 1e-3) / 1e12,
+                "call_list": "optional: homGemmFoldedLayernormF16 in place of GEMM + nvteLayernormF16"}
         del big
+
+    # BERT-base through the optional folded-layer-norm call list (see above)
+    if args.gemm_mode != 0:
+        enc = bert.BertEncoder(d["layers"], d["hidden"], d["heads"], d["ffn"], d["bs"], d["seq"], d["vocab"],
+                               gemm_mode=args.gemm_mode, gelu_form="erf", fold_layernorm=True)
+        enc.load(model)
+        enc.set_inputs(ids=model["ids"], mask=model["mask"])
+        fold_ms = enc.time(args.steps, args.warmup, graph=not args.eager)
+        enc.close()
+        kernels["bert_base_b8_s128_encoder_folded_layernorm"] = {
+            "ms": fold_ms, "sequences/s": d["bs"] / (fold_ms * 1e-3),
+            "call_list": "optional: homGemmFoldedLayernormF16 in place of GEMM + nvteLayernormF16"}
 
     # the reference's whole BertForMaskedLM graph: encoder + LM head to logits [8, 128, 30522]
     enc = bert.BertEncoder(d["layers"], d["hidden"], d["heads"], d["ffn"], d["bs"], d["seq"], d["vocab"],

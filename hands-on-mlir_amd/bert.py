@@ -12,9 +12,14 @@ class BertEncoder:
     ROLES = ("qkv", "out", "ffn1", "ffn2", "transform", "decoder")
 
     def __init__(self, layers, hidden, heads, ffn, bs, seq, vocab, gemm_mode=1, gelu_form="erf",
-                 lm_head=False, role_layout=None):
+                 lm_head=False, role_layout=None, fold_layernorm=False):
         """role_layout: optional {role: "kn" | "nk"} pinning the weight layout (and with it the entry
-        point: cutlassGemmF16 / nvteGemmF16) of individual GEMM roles; others are decided by the driver."""
+        point: cutlassGemmF16 / nvteGemmF16) of individual GEMM roles; others are decided by the driver.
+        fold_layernorm: run the call list whose per-layer layer norms are folded into the GEMMs around them
+        (homGemmFoldedLayernormF16; row-major weights for every role, erf GELU); takes effect in load()."""
+        self.fold_layernorm = fold_layernorm
+        if fold_layernorm:
+            role_layout = dict(role_layout or {}, qkv="kn", out="kn", ffn1="kn", ffn2="kn")
         self.drv = rt.load_driver()
         self.dims = dict(layers=layers, hidden=hidden, heads=heads, ffn=ffn, bs=bs, seq=seq, vocab=vocab)
         self.gemm_mode = gemm_mode
@@ -55,6 +60,10 @@ class BertEncoder:
             # [K, N] operand of the manifest path is word^T and the [N, K] operand of the nvte path is word
             self._upload(0, 6, model["w_transform"].T if nk[4] else model["w_transform"])
             self._upload(0, 7, model["word"] if nk[5] else model["word"].T)
+        if self.fold_layernorm:
+            # (after the uploads: the column sums of Wqkv and W1 are computed from the device copies)
+            if self.drv.homBertFoldLayernorm(self.h) != 0:
+                raise ValueError("the driver refused to fold the layer norms for this configuration")
 
     def set_inputs(self, ids=None, mask=None, hidden=None):
         p = lambda a, dt: (np.ascontiguousarray(a, dt).ctypes.data_as(ctypes.c_void_p)

@@ -83,6 +83,13 @@ struct HomBertEncoder {
   bool lmHead = false;
   Tensor wTransform, wDecoder, t, logits;
   GemmChoice cQkv, cOut, cFfn1, cFfn2, cTransform, cDecoder;
+  // Folded layer norms (homBertFoldLayernorm): the column sums of every Wqkv
+  // and W1 (fp32, device), two buffers of partial row sums that the
+  // residual GEMMs write alternately, and the number of pieces in them.
+  bool foldLn = false;
+  std::vector<float *> colSumQkv, colSumW1;
+  float *rowSums[2] = {nullptr, nullptr};
+  int32_t foldPieces = 0;
   hipStream_t stream = nullptr;
   hipGraph_t graph = nullptr;
   hipGraphExec_t graphExec = nullptr;
@@ -184,6 +191,41 @@ void callList(HomBertEncoder *e, int fromIds) {
   }
   const float scale = 1.0f / sqrtf(float(e->hidden / e->heads));
   const int64_t geluAct = e->gemmMode == 0 ? 1 : (e->geluForm == 1 ? 2 : 1);
+  if (e->foldLn) {
+    // The same graph with the two layer norms of every layer folded into the
+    // GEMMs around them: the residual GEMMs (out-projection, FFN2) leave the
+    // un-normalised sum in h together with the partial row sums of it, and
+    // whoever reads h next -- the following GEMM as its A operand, the next
+    // residual GEMM as its source -- normalises on the fly.  One real layer
+    // norm remains, behind the last layer.  5 launches per layer instead of 7.
+    auto folded = [&](const Tensor &a, const Tensor &w, const Tensor &c,
+                      const Tensor &d, int32_t mode, int64_t act, float beta,
+                      const float *statsIn, const float *colSum,
+                      float *statsOut) {
+      homGemmFoldedLayernormF16(a.m.rank, a.m.descriptor, w.m.rank,
+                                w.m.descriptor, c.m.rank, c.m.descriptor,
+                                d.m.rank, d.m.descriptor, mode, act, 1.0f, beta,
+                                statsIn, e->foldPieces, e->eps, colSum,
+                                statsOut, 0);
+    };
+    const float *stats = nullptr; // h is normalised (embeddings) at the start
+    for (int l = 0; l < e->layers; l++) {
+      const LayerWeights &w = e->w[size_t(l)];
+      folded(e->h, w.wqkv, e->qkv, e->qkv, 1, 0, 0.0f, stats,
+             e->colSumQkv[size_t(l)], nullptr);
+      nvteBertAttentionF16(e->qkv.m.rank, e->qkv.m.descriptor, e->cu.m.rank,
+                           e->cu.m.descriptor, e->attn.m.rank,
+                           e->attn.m.descriptor, scale, e->heads);
+      folded(e->attn, w.wo, e->h, e->h, 2, 0, 1.0f, stats, nullptr,
+             e->rowSums[0]);
+      folded(e->h, w.w1, e->f, e->f, 1, 1, 0.0f, e->rowSums[0],
+             e->colSumW1[size_t(l)], nullptr);
+      folded(e->f, w.w2, e->h, e->h, 2, 0, 1.0f, e->rowSums[0], nullptr,
+             e->rowSums[1]);
+      stats = e->rowSums[1];
+    }
+    nvteLayernormF16(e->h.m.rank, e->h.m.descriptor, e->eps);
+  } else
   for (int l = 0; l < e->layers; l++) {
     const LayerWeights &w = e->w[l];
     gemm(e, e->h, w.wqkv, e->qkv, e->qkv, 0, 0.0f, e->cQkv);
@@ -318,6 +360,57 @@ DRV_EXPORT int homBertEnableLmHead(HomBertEncoder *e) {
   return 0;
 }
 
+// Switches the call list to the variant with folded layer norms (see
+// callList).  Call after every weight has been uploaded (the column sums of
+// Wqkv and W1 are computed here) and before capturing a graph.  Needs all four
+// GEMM roles on row-major weights and the erf form of GELU; the LM head keeps
+// its own layer norm.  Returns 0, or -1 when the configuration does not allow
+// it (nothing changes then).
+DRV_EXPORT int homBertFoldLayernorm(HomBertEncoder *e) {
+  if (e->foldLn)
+    return 0;
+  if (e->cQkv.nk || e->cOut.nk || e->cFfn1.nk || e->cFfn2.nk ||
+      e->geluForm != 0 || e->gemmMode == 0 || e->hidden % 8 != 0 ||
+      e->ffn % 8 != 0) {
+    fprintf(stderr, "hom_bert_driver: folded layer norms need row-major "
+                    "weights for every GEMM role and the erf form of GELU\n");
+    return -1;
+  }
+  const int64_t M = int64_t(e->batch) * e->seq;
+  const int32_t pOut = homFoldedLayernormPieces(M, e->hidden, e->hidden, 0, 0);
+  const int32_t pFfn2 = homFoldedLayernormPieces(M, e->hidden, e->ffn, 0, 0);
+  if (pOut != pFfn2 || pOut < 1)
+    return -1; // (both depend on M and N only)
+  bool ok = true;
+  for (float *&q : e->rowSums)
+    ok = ok && hipOk(hipMalloc(reinterpret_cast<void **>(&q),
+                               size_t(pOut) * size_t(M) * 2 * sizeof(float)),
+                     "hipMalloc");
+  void *prev = homGetStream();
+  homSetStream(e->stream);
+  for (int l = 0; l < e->layers && ok; l++) {
+    float *q = nullptr, *f = nullptr;
+    ok = hipOk(hipMalloc(reinterpret_cast<void **>(&q), size_t(3) * e->hidden * 4),
+               "hipMalloc") &&
+         hipOk(hipMalloc(reinterpret_cast<void **>(&f), size_t(e->ffn) * 4),
+               "hipMalloc");
+    e->colSumQkv.push_back(q);
+    e->colSumW1.push_back(f);
+    if (ok) {
+      const LayerWeights &w = e->w[size_t(l)];
+      homColumnSumsF16(w.wqkv.m.rank, w.wqkv.m.descriptor, q);
+      homColumnSumsF16(w.w1.m.rank, w.w1.m.descriptor, f);
+    }
+  }
+  homSetStream(prev);
+  ok = ok && hipOk(hipStreamSynchronize(e->stream), "hipStreamSynchronize");
+  if (!ok)
+    return -1;
+  e->foldPieces = pOut;
+  e->foldLn = true;
+  return 0;
+}
+
 DRV_EXPORT void homBertDestroy(HomBertEncoder *e) {
   if (!e)
     return;
@@ -339,6 +432,13 @@ DRV_EXPORT void homBertDestroy(HomBertEncoder *e) {
     w.w1.release();
     w.w2.release();
   }
+  for (float *q : e->colSumQkv)
+    (void)hipFree(q);
+  for (float *q : e->colSumW1)
+    (void)hipFree(q);
+  for (float *q : e->rowSums)
+    if (q)
+      (void)hipFree(q);
   for (Tensor *t : {&e->wordEmb, &e->posType, &e->ids, &e->mask, &e->cu, &e->h,
                     &e->emb, &e->qkv, &e->attn, &e->f, &e->wTransform,
                     &e->wDecoder, &e->t, &e->logits})

@@ -94,6 +94,14 @@ struct GemmParams {
   const _Float16 *rowShift;
   const float *colSum;
   int colSumSlices;
+  // folded layer norm (kEpiFold* kernels only): partial (sum, sum of squares)
+  // pairs [foldPieces][M] of the rows a layer norm is folded away from -- the
+  // rows of A (kEpiFoldA, kEpiFoldAGelu) or of C (kEpiFoldCStats) -- the
+  // reciprocal of their length and the layer norm's epsilon.  Null: the rows
+  // are used as they are.
+  const float *foldStats;
+  int foldPieces;
+  float foldInvN, foldEps;
 };
 
 // Epilogue codes beyond the three activations of the manifest kernels: linear
@@ -101,6 +109,18 @@ struct GemmParams {
 // affine transform of A folded into the accumulator.
 constexpr int kEpiRowStats = 3;
 constexpr int kEpiRowAffine = 4;
+// A layer norm (no affine parameters) folded into the GEMMs on either side of
+// it, with its statistics travelling as the fp32 partial sums that the
+// producing GEMM's epilogue wrote (nothing in between):
+//   kEpiFoldA       D = alpha (LN(A) . B) + beta C
+//   kEpiFoldAGelu   D = GELU_erf(alpha (LN(A) . B) + beta C)
+//   kEpiFoldCStats  D = alpha (A . B) + beta LN(C), plus the partial sums of
+//                   the stored D (for the next folded layer norm)
+// LN(A) . B is evaluated as rstd_m (A . B) - mu_m rstd_m colsum(B), see
+// kEpiRowAffine.
+constexpr int kEpiFoldA = 5;
+constexpr int kEpiFoldAGelu = 6;
+constexpr int kEpiFoldCStats = 7;
 
 // GELU(x) = 0.5 x (1 + erf(x / sqrt 2)) = max(x, 0) - 0.5 |x| erfc(|x| / sqrt 2)
 // (x >= 0: 1 + erf = 2 - erfc; x < 0: 1 + erf = erfc(|z|); no cancellation on
@@ -520,6 +540,234 @@ epilogueFast(const GemmParams &p, float16v (&acc)[MI][NI], int m0, int n0,
 }
 
 
+// (rstd, -mean * rstd) of row m0 + tid of a folded layer norm, for the first BM
+// threads of the workgroup, in two steps: foldRowStatRequest asks for the
+// row's first pieces (no branch around a load: an index past the last piece
+// re-reads the last piece, so the batch is one memory round trip) and
+// foldRowStatFinish adds them up (pieces beyond the batch, which no BERT shape
+// has, are fetched there).  The kernels request next to their first slab loads; the
+// round trip then overlaps the main loop (tiles with registers to spare keep
+// those pairs until the epilogue) or the wait for the first slab (256-row
+// tiles finish at once).  kFoldBatch: pieces requested up front, sized for rows
+// of up to 1024 columns (BERT's hidden sizes) cut into tiles BM wide.
+template <int BM> struct FoldBatch {
+  static constexpr int value = BM >= 256 ? 4 : (BM >= 128 ? 8 : 16);
+};
+template <int BM>
+__device__ __forceinline__ void
+foldRowStatRequest(const GemmParams &p, int m0, int tid,
+                   float2v (&v)[FoldBatch<BM>::value]) {
+  constexpr int kFoldBatch = FoldBatch<BM>::value;
+  // Every thread loads, from an address that is always valid, so that nothing
+  // stands between these requests and the ones around them: threads past the
+  // tile's rows repeat a row, and without statistics the first bytes of A's
+  // rows are read (and ignored by foldRowStatFinish).
+  const bool folded = p.foldStats != nullptr;
+  const float *base =
+      folded ? p.foldStats : reinterpret_cast<const float *>(p.A);
+  const int pieces = folded ? p.foldPieces : 1;
+  const int row = m0 + (tid < BM ? tid : 0);
+  const int m = row < p.M ? row : p.M - 1;
+#pragma unroll
+  for (int u = 0; u < kFoldBatch; u++) {
+    const int at = u < pieces ? u : pieces - 1;
+    v[u] = *reinterpret_cast<const float2v *>(base +
+                                              (int64_t(at) * p.M + m) * 2);
+  }
+}
+template <int BM>
+__device__ __forceinline__ float2v
+foldRowStatFinish(const GemmParams &p, int m0, int tid,
+                  const float2v (&v)[FoldBatch<BM>::value]) {
+  constexpr int kFoldBatch = FoldBatch<BM>::value;
+  float2v stat{1.f, 0.f};
+  if (p.foldStats != nullptr && tid < BM) {
+    const int m = m0 + tid < p.M ? m0 + tid : p.M - 1;
+    float s = 0.f, sq = 0.f;
+#pragma unroll
+    for (int u = 0; u < kFoldBatch; u++) {
+      s += u < p.foldPieces ? v[u][0] : 0.f;
+      sq += u < p.foldPieces ? v[u][1] : 0.f;
+    }
+    for (int pc = kFoldBatch; pc < p.foldPieces; pc++) {
+      const float2v w = *reinterpret_cast<const float2v *>(
+          p.foldStats + (int64_t(pc) * p.M + m) * 2);
+      s += w[0];
+      sq += w[1];
+    }
+    const float mu = s * p.foldInvN;
+    // the difference cancels to a small negative number for near-constant
+    // rows; clamped so that a tiny eps cannot turn it into a NaN
+    const float rstd =
+        1.0f / sqrtf(fmaxf(sq * p.foldInvN - mu * mu, 0.f) + p.foldEps);
+    stat[0] = rstd;
+    stat[1] = -mu * rstd;
+  }
+  return stat;
+}
+
+// The epilogues with a folded layer norm (kEpiFold*).  Same memory access
+// scheme as epilogueFast (buffer descriptors per wavefront, 16-byte accesses,
+// every source vector requested before the transposition): N, ldd and ldc
+// multiples of 8, C / D 16-byte aligned, C absent or a full [M, N] matrix; the
+// host checks this.  myStat: foldRowStat() of this thread's row; the pairs of
+// the workgroup's BM rows meet in LDS, behind the wavefronts' accumulator
+// strips.
+template <int MI, int NI, int WTM, int WTN, int EPI, int BM, int THREADS>
+__device__ __forceinline__ void
+epilogueFold(const GemmParams &p, float16v (&acc)[MI][NI], int m0, int n0,
+             int waveM, int waveN, int lane, int wave, int tid,
+             float2v myStat, unsigned char *smem) {
+  constexpr bool kFoldA = EPI == kEpiFoldA || EPI == kEpiFoldAGelu;
+  constexpr bool kFoldC = EPI == kEpiFoldCStats;
+  constexpr bool kStats = EPI == kEpiFoldCStats;
+  constexpr int ROW_B = WTN * 4 + 16;
+  constexpr int LPR = WTN / 8;  // lanes per row on the way out
+  constexpr int RPP = 64 / LPR; // rows per pass
+  constexpr int PASSES = 32 / RPP;
+  static_assert(RPP * LPR == 64 && PASSES * RPP == 32,
+                "folded epilogues need a power-of-two wave tile width");
+  constexpr uint32_t kOob = 0x80000000u;
+  constexpr int kStripBytes = (THREADS / kWave) * 32 * ROW_B;
+  constexpr int WN_ = (THREADS / kWave) / (BM / WTM); // wavefront columns
+  unsigned char *mine = smem + wave * (32 * ROW_B);
+  float2v *rowStat = reinterpret_cast<float2v *>(smem + kStripBytes);
+  // (kStats) partial sums of the tile's rows per wavefront column, [BM][WN]
+  float2v *tileSums = rowStat + BM;
+  const int l32 = lane % 32, kb = lane / 32;
+  const int rr = lane / LPR, cc = (lane % LPR) * 8;
+  const int rowBase = m0 + waveM * WTM;
+  const int colBase = n0 + waveN * WTN;
+  const int n = colBase + cc;
+  auto clampBytes = [](int64_t b) -> int32_t {
+    return b > 0x7fffffffLL ? 0x7fffffff : (b < 0 ? 0 : int32_t(b));
+  };
+  const int rowsLeft = p.M - rowBase;
+  const auto rsrcD = __builtin_amdgcn_make_buffer_rsrc(
+      p.D + int64_t(rowBase) * p.ldd + colBase, 0,
+      clampBytes((int64_t(rowsLeft) * p.ldd - colBase) * 2), 0x00020000);
+  const uint32_t ldd2 = uint32_t(p.ldd) * 2u, ldc2 = uint32_t(p.ldc) * 2u;
+  const uint32_t colOff = n < p.N ? uint32_t(cc) * 2u : kOob;
+  typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+  const bool useC = p.beta != 0.f;
+  const bool folded = p.foldStats != nullptr;
+  // column sums of B for this lane's 8 columns (the same in every pass)
+  float cs[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  if constexpr (kFoldA) {
+    if (folded && n < p.N) {
+      const float4v *src = reinterpret_cast<const float4v *>(p.colSum + n);
+      const float4v a = src[0], b = src[1];
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        cs[e] = a[e];
+        cs[e + 4] = b[e];
+      }
+    }
+  }
+  half8 cv[MI][PASSES];
+  if (useC) {
+    const auto rsrcC = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<_Float16 *>(p.C) + int64_t(rowBase) * p.ldc + colBase, 0,
+        clampBytes((int64_t(rowsLeft) * p.ldc - colBase) * 2), 0x00020000);
+#pragma unroll
+    for (int i = 0; i < MI; i++)
+#pragma unroll
+      for (int ps = 0; ps < PASSES; ps++) {
+        const uint32_t r = uint32_t(i * 32 + ps * RPP + rr);
+        cv[i][ps] = __builtin_bit_cast(
+            half8, __builtin_amdgcn_raw_buffer_load_b128(
+                       rsrcC, colOff == kOob ? kOob : r * ldc2 + colOff, 0, 0));
+      }
+  }
+  __syncthreads(); // no wavefront still reads operands from the main loop's LDS
+  if (tid < BM)
+    rowStat[tid] = myStat;
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < MI; i++) {
+#pragma unroll
+    for (int j = 0; j < NI; j++)
+#pragma unroll
+      for (int g = 0; g < 4; g++) {
+        float4v v;
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+          v[e] = acc[i][j][g * 4 + e];
+        *reinterpret_cast<float4v *>(mine + l32 * ROW_B +
+                                     (j * 32 + g * 8 + kb * 4) * 4) = v;
+      }
+#pragma unroll
+    for (int ps = 0; ps < PASSES; ps++) {
+      const int r = ps * RPP + rr;
+      const float4v lo =
+          *reinterpret_cast<const float4v *>(mine + r * ROW_B + cc * 4);
+      const float4v hi =
+          *reinterpret_cast<const float4v *>(mine + r * ROW_B + cc * 4 + 16);
+      const float2v st = rowStat[waveM * WTM + i * 32 + r];
+      half8 o;
+      float rowSum = 0.f, rowSq = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; e++) {
+        float a = e < 4 ? lo[e] : hi[e - 4];
+        if constexpr (kFoldA)
+          a = fmaf(st[0], a, st[1] * cs[e]);
+        float v = p.alpha * a;
+        if (useC) {
+          float c = float(cv[i][ps][e]);
+          if constexpr (kFoldC)
+            c = fmaf(c, st[0], st[1]);
+          v = fmaf(p.beta, c, v);
+        }
+        if constexpr (EPI == kEpiFoldAGelu)
+          v = geluErf(v);
+        o[e] = _Float16(v);
+        if constexpr (kStats) {
+          // statistics of the values as stored
+          const float x = float(o[e]);
+          rowSum += x;
+          rowSq = fmaf(x, x, rowSq);
+        }
+      }
+      const uint32_t row = uint32_t(i * 32 + r);
+      __builtin_amdgcn_raw_buffer_store_b128(
+          __builtin_bit_cast(u32x4, o), rsrcD,
+          colOff == kOob ? kOob : row * ldd2 + colOff, 0, kWriteThroughAux);
+      if constexpr (kStats) {
+        // the LPR lanes of a row hold its WTN columns (columns past N
+        // contribute nothing); the wavefront columns of the tile meet in LDS
+        if (colOff == kOob)
+          rowSum = rowSq = 0.f;
+        rowSum = sumAcrossLanes<LPR>(rowSum);
+        rowSq = sumAcrossLanes<LPR>(rowSq);
+        if (lane % LPR == 0) {
+          float2v out;
+          out[0] = rowSum;
+          out[1] = rowSq;
+          tileSums[(waveM * WTM + int(row)) * WN_ + waveN] = out;
+        }
+      }
+    }
+  }
+  if constexpr (kStats) {
+    // one (sum, sum of squares) pair per row and tile column: piece n0 / BN
+    __syncthreads();
+    if (tid < BM && m0 + tid < p.M) {
+      float2v out{0.f, 0.f};
+#pragma unroll
+      for (int w = 0; w < WN_; w++) {
+        out[0] += tileSums[tid * WN_ + w][0];
+        out[1] += tileSums[tid * WN_ + w][1];
+      }
+      const int piece = n0 / (WTN * WN_);
+      // (written through: the next kernel reads them first thing)
+      storeWriteThrough(reinterpret_cast<float2v *>(
+                            p.rowStatPartials +
+                            (int64_t(piece) * p.M + m0 + tid) * 2),
+                        out);
+    }
+  }
+}
+
 // Whether epilogueFast applies (wave-uniform), and with which source mode
 // (0 none, 1 bias row, 2 full matrix); -1 = use epilogueStoreLds.
 __host__ __device__ __forceinline__ int epilogueFastMode(const GemmParams &p,
@@ -548,6 +796,7 @@ template <int MI, int NI, int WTM, int WTN, int EPI>
 __device__ __forceinline__ void
 epilogueAuto(const GemmParams &p, float16v (&acc)[MI][NI], int m0, int n0,
              int waveM, int waveN, int lane, int wave, unsigned char *smem) {
+  static_assert(EPI < kEpiFoldA, "folded epilogues are called directly");
   if constexpr (EPI <= int(Epilogue::kGeluTanh)) {
     const int mode = p.epiMode;
     if (mode == 0)
@@ -756,6 +1005,10 @@ Status planLaunch(const GemmProblem &pr, LaunchPlan *plan) {
   p.rowShift = pr.rowShift;
   p.colSum = pr.colSum;
   p.colSumSlices = pr.colSumSlices;
+  p.foldStats = pr.foldStats;
+  p.foldPieces = pr.foldPieces;
+  p.foldInvN = pr.foldInvN;
+  p.foldEps = pr.foldEps;
   p.tilesM = int((pr.M + BM - 1) / BM);
   p.tilesN = int((pr.N + BN - 1) / BN);
   const int kTiles = int((pr.K + BK - 1) / BK);

@@ -114,13 +114,16 @@ FusedTile fusedTileFor(int likeKernel) {
 }
 template <int EPI>
 Status launchFusedTile(int likeKernel, const GemmProblem &p, hipStream_t s) {
+  // the folded-layer-norm epilogues run on the DMA-staged variants of the two
+  // smaller tiles (the faster ones at the sizes those tiles serve)
+  constexpr bool kDma = EPI >= kEpiFoldA;
   switch (fusedTileFor(likeKernel).edge) {
   case 256:
     return launchPipe<256, 256, 2, 4, 1, EPI, false>(p, s);
   case 128:
-    return launchPipe<128, 128, 2, 4, 2, EPI, false>(p, s);
+    return launchPipe<128, 128, 2, 4, kDma ? 3 : 2, EPI, false, kDma>(p, s);
   default:
-    return launchPipe<64, 64, 2, 2, 2, EPI, false>(p, s);
+    return launchPipe<64, 64, 2, 2, kDma ? 3 : 2, EPI, false, kDma>(p, s);
   }
 }
 
@@ -191,6 +194,63 @@ Status launchGemmRowAffine(int likeKernel, const GemmProblem &p,
   q.colSum = colSum;
   q.colSumSlices = slices;
   return launchFusedTile<kEpiRowAffine>(likeKernel, q, s);
+}
+
+int foldedPieces(int likeKernel, int64_t N) {
+  // one piece per tile column (the wavefront columns of a tile are added up
+  // inside the workgroup)
+  const FusedTile t = fusedTileFor(likeKernel);
+  return int((N + t.edge - 1) / t.edge);
+}
+
+Status launchColumnSums(const _Float16 *B, int64_t ldb, int64_t K, int64_t N,
+                        float *out, hipStream_t s) {
+  HOM_CHECK_RET(K > 0 && N > 0 && K < (int64_t(1) << 31) &&
+                    N < (int64_t(1) << 31) && N % 8 == 0 && ldb % 8 == 0 &&
+                    aligned16(B),
+                Status::kInvalidArgument,
+                "column sums: N and the leading dimension must be multiples of 8");
+  colSumKernel<<<dim3((unsigned)((N + 31) / 32), 1), dim3(256), 0, s>>>(
+      B, ldb, int(K), int(N), int(K), out);
+  HOM_HIP_RET(hipGetLastError(), Status::kInternal);
+  return Status::kSuccess;
+}
+
+Status launchGemmFolded(int likeKernel, const GemmProblem &p, int mode,
+                        int activation, float *statsOut, hipStream_t s) {
+  HOM_CHECK_RET(likeKernel >= 0 && likeKernel < gemmKernelCount() &&
+                    fusedGemmFits(p) &&
+                    (p.beta == 0.f || (p.cRowPeriod >= p.M && p.ldc % 8 == 0)),
+                Status::kInvalidArgument,
+                "folded layer norm + gemm: problem does not fit the fused kernels");
+  HOM_CHECK_RET((mode == 1 && (activation == 0 || activation == 1) && !statsOut &&
+                 (!p.foldStats || p.colSum)) ||
+                    (mode == 2 && activation == 0 &&
+                     (!p.foldStats || p.beta != 0.f)),
+                Status::kInvalidArgument,
+                "folded layer norm + gemm: mode %d / activation %d not supported",
+                mode, activation);
+  // 32-bit byte offsets inside a tile's rows
+  HOM_CHECK_RET(int64_t(256) * p.ldd * 2 < (int64_t(1) << 31) &&
+                    int64_t(256) * p.ldc * 2 < (int64_t(1) << 31),
+                Status::kInvalidArgument,
+                "folded layer norm + gemm: leading dimension too large");
+  GemmProblem q = p;
+  q.splitK = 1;
+  q.colSumSlices = 1;
+  q.rowStatPartials = statsOut;
+  if (mode == 1)
+    return activation == 1 ? launchFusedTile<kEpiFoldAGelu>(likeKernel, q, s)
+                           : launchFusedTile<kEpiFoldA>(likeKernel, q, s);
+  if (!statsOut) {
+    // the kernel always writes its partial sums: give it somewhere to put them
+    const size_t bytes =
+        size_t(foldedPieces(likeKernel, p.N)) * size_t(p.M) * 2 * sizeof(float);
+    q.rowStatPartials = static_cast<float *>(libraryScratch(kTemp, bytes, false));
+    if (!q.rowStatPartials)
+      return Status::kInternal;
+  }
+  return launchFusedTile<kEpiFoldCStats>(likeKernel, q, s);
 }
 
 } // namespace hom

@@ -94,6 +94,12 @@ struct GemmProblem {
   const _Float16 *rowShift;
   const float *colSum;
   int colSumSlices;
+  // Folded layer norm, used by launchGemmFolded only (null otherwise): the
+  // partial (sum, sum of squares) pairs [foldPieces][M] of the rows that a
+  // layer norm is folded away from, 1 / their length, the epsilon.
+  const float *foldStats;
+  int foldPieces;
+  float foldInvN, foldEps;
 };
 
 struct GemmKernelInfo {
@@ -135,5 +141,22 @@ Status launchGemmRowStats(int likeKernel, const GemmProblem &p, _Float16 *var,
 Status launchGemmRowAffine(int likeKernel, const GemmProblem &p,
                            const _Float16 *var, const _Float16 *mean,
                            hipStream_t s);
+
+// A layer norm without affine parameters folded into the GEMMs around it (no
+// counterpart in the reference, whose pair exchanges finished fp16 statistics
+// through two more kernels).  mode 1: D = act(alpha LN(A) B + beta C), act =
+// linear or GELU-erf (activation 0 / 1); mode 2: D = alpha A B + beta LN(C).
+// The statistics of the normalised rows arrive as the partial sums an earlier
+// launchGemmFolded wrote (p.foldStats / foldPieces / foldInvN / foldEps; null:
+// no normalisation); mode 1 also needs the column sums of B (p.colSum, one
+// slice, see launchColumnSums).  statsOut != null (mode 2 only): the partial
+// sums of the stored D go there, foldedPieces(likeKernel, N) x M pairs.
+// Needs the alignment class of fusedGemmFits and C absent or a full matrix.
+Status launchGemmFolded(int likeKernel, const GemmProblem &p, int mode,
+                        int activation, float *statsOut, hipStream_t s);
+int foldedPieces(int likeKernel, int64_t N);
+// out[n] = sum over k of B[k, n] (fp32), B row-major [K, N], N % 8 == 0.
+Status launchColumnSums(const _Float16 *B, int64_t ldb, int64_t K, int64_t N,
+                        float *out, hipStream_t s);
 
 } // namespace hom

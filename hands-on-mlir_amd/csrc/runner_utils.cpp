@@ -199,6 +199,27 @@ void homAddLayernormF16(int64_t rankX, void *dstX, int64_t rankRes,
                            rankBeta, dstBeta, rankOut, dstOut, eps);
 }
 
+void homGemmFoldedLayernormF16(int64_t rankA, void *dstA, int64_t rankB,
+                               void *dstB, int64_t rankC, void *dstC,
+                               int64_t rankD, void *dstD, int32_t mode,
+                               int64_t activation, float alpha, float beta,
+                               const float *statsIn, int32_t piecesIn, float eps,
+                               const float *colSumB, float *statsOut,
+                               int32_t likeGemmNum) {
+  (void)runGemmFoldedLayernorm(rankA, dstA, rankB, dstB, rankC, dstC, rankD,
+                               dstD, mode, activation, alpha, beta, statsIn,
+                               piecesIn, eps, colSumB, statsOut, likeGemmNum);
+}
+
+int32_t homFoldedLayernormPieces(int64_t M, int64_t N, int64_t K,
+                                 int64_t activation, int32_t likeGemmNum) {
+  return foldedLayernormPieces(M, N, K, activation, likeGemmNum);
+}
+
+void homColumnSumsF16(int64_t rankB, void *dstB, float *out) {
+  (void)runColumnSums(rankB, dstB, out);
+}
+
 void homGeluF16(int64_t rankA, void *dstA, int64_t rankOut, void *dstOut,
                 int32_t form) {
   (void)runGeluF16(rankA, dstA, rankOut, dstOut, form);

@@ -468,6 +468,76 @@ Status runGemmWithVarMean(int64_t rankA, void *dstA, int64_t rankB, void *dstB,
   return launchRowStatsF16(D.data, Var.data, Mean.data, rows, n, eps, stream());
 }
 
+namespace {
+// The tile family member a folded GEMM imitates: the caller's manifest kernel
+// (1-based) or the library's choice for the shape.
+int foldedLikeKernel(const GemmProblem &pr, int64_t activation, int32_t likeGemmNum) {
+  (void)activation;
+  if (likeGemmNum >= 1 && likeGemmNum <= gemmKernelCount())
+    return likeGemmNum - 1;
+  // The folded kernels exist with 256 x 256, 128 x 128 and 64 x 64 tiles: the
+  // largest that still gives most of the CUs a tile.
+  auto tiles = [&](int64_t edge) {
+    return ((pr.M + edge - 1) / edge) * ((pr.N + edge - 1) / edge);
+  };
+  const int cus = deviceInfo().computeUnits > 0 ? deviceInfo().computeUnits : 256;
+  const int edge = tiles(256) * 5 >= int64_t(cus) * 4   ? 256
+                   : tiles(128) * 2 >= int64_t(cus) ? 128
+                                                    : 64;
+  const int like = findKernel(edge, edge, 64, Epilogue::kLinear, 8);
+  return like >= 0 ? like : 0;
+}
+} // namespace
+
+Status runGemmFoldedLayernorm(int64_t rankA, void *dstA, int64_t rankB,
+                              void *dstB, int64_t rankC, void *dstC,
+                              int64_t rankD, void *dstD, int32_t mode,
+                              int64_t activation, float alpha, float beta,
+                              const float *statsIn, int32_t piecesIn, float eps,
+                              const float *colSumB, float *statsOut,
+                              int32_t likeGemmNum) {
+  View<_Float16> A(rankA, dstA), B(rankB, dstB), C(rankC, dstC), D(rankD, dstD);
+  GemmProblem pr{};
+  GemmShapes sh{};
+  Status st = checkGemmOperands(A, B, C, D, false, beta, &sh, &pr);
+  if (st != Status::kSuccess)
+    return st;
+  HOM_CHECK_RET(mode == 1 || mode == 2, Status::kInvalidArgument,
+                "folded layer norm: mode must be 1 (rows of A) or 2 (rows of C), got %d",
+                mode);
+  HOM_CHECK_RET(!statsIn || piecesIn >= 1, Status::kInvalidArgument,
+                "folded layer norm: %d pieces of partial sums", piecesIn);
+  pr.alpha = alpha;
+  pr.beta = beta;
+  pr.foldStats = statsIn;
+  pr.foldPieces = piecesIn;
+  pr.foldInvN = 1.0f / float(mode == 1 ? pr.K : pr.N);
+  pr.foldEps = eps;
+  pr.colSum = colSumB;
+  if (pr.M == 0 || pr.N == 0)
+    return Status::kSuccess;
+  return launchGemmFolded(foldedLikeKernel(pr, activation, likeGemmNum), pr, mode,
+                          int(activation), statsOut, stream());
+}
+
+int32_t foldedLayernormPieces(int64_t M, int64_t N, int64_t K, int64_t activation,
+                              int32_t likeGemmNum) {
+  GemmProblem pr{};
+  pr.M = M;
+  pr.N = N;
+  pr.K = K;
+  return foldedPieces(foldedLikeKernel(pr, activation, likeGemmNum), N);
+}
+
+Status runColumnSums(int64_t rankB, void *dstB, float *out) {
+  View<_Float16> B(rankB, dstB);
+  HOM_CHECK_RET(B.sizes && rankB == 3 && B.sizes[0] == 1 && B.strides[2] == 1,
+                Status::kInvalidArgument,
+                "column sums: B must be a [1, K, N] tensor with contiguous rows");
+  return launchColumnSums(B.data, B.strides[1], B.sizes[1], B.sizes[2], out,
+                          stream());
+}
+
 Status runLayernormGemm(int64_t rankA, void *dstA, int64_t rankB, void *dstB,
                         int64_t rankC, void *dstC, int64_t rankD, void *dstD,
                         int64_t rankVar, void *dstVar, int64_t rankMean,

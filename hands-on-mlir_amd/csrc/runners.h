@@ -34,6 +34,19 @@ Status runLayernormGemm(int64_t rankA, void *dstA, int64_t rankB, void *dstB,
                         void *dstMean, float alpha, float beta,
                         int64_t activation);
 
+// GEMM with a layer norm (no affine parameters) of the rows of A (mode 1) or
+// of C (mode 2) folded in; see launchGemmFolded.
+Status runGemmFoldedLayernorm(int64_t rankA, void *dstA, int64_t rankB,
+                              void *dstB, int64_t rankC, void *dstC,
+                              int64_t rankD, void *dstD, int32_t mode,
+                              int64_t activation, float alpha, float beta,
+                              const float *statsIn, int32_t piecesIn, float eps,
+                              const float *colSumB, float *statsOut,
+                              int32_t likeGemmNum);
+int32_t foldedLayernormPieces(int64_t M, int64_t N, int64_t K, int64_t activation,
+                              int32_t likeGemmNum);
+Status runColumnSums(int64_t rankB, void *dstB, float *out);
+
 // Kernel choice without timing: tuned table first, heuristic otherwise.
 // `activation`: 0 linear, 1 GELU (erf), 2 GELU (tanh).  Returns true when the
 // shape was found in the tuned table.

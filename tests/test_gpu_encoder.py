@@ -341,6 +341,68 @@ def test_bert_base_b8_s128(gpu, oracle, synth):
         enc.close()
 
 
+def test_folded_layernorm_encoder(gpu, oracle, synth):
+    """The optional call list with every per-layer layer norm folded into the GEMMs around it
+    (homGemmFoldedLayernormF16: 5 launches per layer instead of 7) computes the same encoder: a small model
+    eagerly and as a replayed graph, then BERT-base b8 x s128 against both oracles with the bounds of the
+    reference call list.  (The normalised hidden states are never rounded to fp16 in this mode, so it sits a
+    little closer to the fp32 reference than the fp16-faithful oracle does.)"""
+    bert = importlib.import_module("hands-on-mlir_amd.bert")
+    model = synth.bert_encoder(layers=3, hidden=128, heads=2, ffn=512, bs=3, seq=64, vocab=1000, config=40)
+    model["lens"][:] = [64, 17, 33]
+    model["mask"] = synth.mask_from_lengths(model["lens"], 64)
+    want = oracle_forward(oracle, model, "erf")
+    enc = bert.BertEncoder(3, 128, 2, 512, 3, 64, 1000, gemm_mode=1, gelu_form="erf", fold_layernorm=True)
+    try:
+        enc.load(model)
+        enc.set_inputs(ids=model["ids"], mask=model["mask"])
+        enc.forward()
+        eager = enc.output()
+        check(eager, want, model["lens"], "folded layer norms, small encoder")
+        enc.capture()
+        for _ in range(3):
+            enc.replay()
+            assert np.array_equal(enc.output(), eager)
+            enc.forward()
+            assert np.array_equal(enc.output(), eager)
+    finally:
+        enc.close()
+    with pytest.raises(ValueError):      # the folded FFN1 epilogue computes the erf form only
+        bert.BertEncoder(3, 128, 2, 512, 3, 64, 1000, gemm_mode=1, gelu_form="tanh", fold_layernorm=True).load(model)
+
+    model = synth.bert_encoder()
+    d = model["dims"]
+    enc = bert.BertEncoder(d["layers"], d["hidden"], d["heads"], d["ffn"], d["bs"], d["seq"], d["vocab"],
+                           gemm_mode=1, gelu_form="erf", fold_layernorm=True)
+    try:
+        enc.load(model)
+        enc.set_inputs(ids=model["ids"], mask=model["mask"])
+        enc.capture()
+        enc.replay()
+        got = enc.output()
+    finally:
+        enc.close()
+    faithful = oracle_forward(oracle, model, "erf")
+    pure = oracle_forward(oracle, model, "erf", round_intermediates=False)
+    # Against the fp16-faithful oracle this mode is a second fp16 pipeline with rounding points of its own
+    # (it never rounds the normalised states), so the two drift apart by the noise of both.  An element
+    # further apart than the bound is at least half the bound away from the fp32 reference in one of the two
+    # pipelines: that count is the allowance.
+    half = (outliers(got, pure, model["lens"], atol=5e-3, rtol=5e-4)[0] +
+            outliers(faithful.astype(np.float16), pure, model["lens"], atol=5e-3, rtol=5e-4)[0])
+    rel16 = check(got, faithful, model["lens"], "folded BERT-base vs fp16-faithful oracle", rel_limit=2e-3,
+                  allowed_outliers=half)
+    floor_out, _ = outliers(faithful.astype(np.float16), pure, model["lens"])
+    gpu_out, gpu_worst = outliers(got, pure, model["lens"])
+    floor = relerr(faithful.astype(np.float16), pure, model["lens"])
+    rel32 = check(got, pure, model["lens"], "folded BERT-base vs fp32 reference", rel_limit=2e-3,
+                  allowed_outliers=floor_out + 1)
+    print(f"folded layer norms, BERT-base: {rel16:.3e} vs fp16-faithful oracle, {rel32:.3e} vs fp32 reference "
+          f"(fp16-storage floor {floor:.3e}); elements outside rtol 1e-3 / atol 1e-2 of the fp32 reference: "
+          f"{gpu_out} (oracle's fp16 pipeline: {floor_out})")
+    assert rel32 <= 1.1 * floor
+
+
 def test_single_layer_full_width(gpu, oracle, synth):
     """One BERT-base layer from identical inputs: no drift yet, so the single-op
     bound holds end to end (norm-wise <= 1e-3, elementwise rtol 1e-3 / atol 1e-2)."""

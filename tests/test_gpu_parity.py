@@ -486,6 +486,75 @@ def test_ln_gemm_pair_constant_rows_stay_finite(gpu, rt):
         assert (v > 0).all()
 
 
+@pytest.mark.parametrize("Mp,H,F,tile", [
+    (1024, 768, 3072, None),                  # BERT-base sizes, library-chosen tiles
+    (200, 264, 520, "64x64_64x2r2_w2x2"),     # ragged rows and columns (multiples of 8)
+    (300, 264, 520, "128x128_64x2r2_w2x4"),
+    (520, 520, 264, "256x256_64x2r1_w2x4"),
+])
+def test_folded_layernorm_gemm_chain(gpu, rt, oracle, Mp, H, F, tile):
+    """x1 = a . Wo + r (+ partial row sums); f = GELU(LN(x1) . W1); x2 = f . W2 + LN(x1) (+ partial row sums);
+    q = LN(x2) . Wq: the post-LN transformer block with both layer norms folded into the GEMMs around them
+    (homGemmFoldedLayernormF16).  Every product is checked against fp64 arithmetic on the fp16 tensors the GPU
+    stored, with the layer norm in its closed form (pinned for the oracle by test_oracle.py)."""
+    M = rt.MemRef.from_tensor
+    g = np.random.default_rng(Mp + H + F)
+    eps = 1e-12
+    num = knum(rt, tile) if tile else 0
+    a = g.standard_normal((1, Mp, H)).astype(np.float16)
+    wo = (g.standard_normal((1, H, H)) * 0.05).astype(np.float16)
+    w1 = (g.standard_normal((1, H, F)) * 0.05).astype(np.float16)
+    w2 = (g.standard_normal((1, F, H)) * 0.05).astype(np.float16)
+    wq = (g.standard_normal((1, H, 3 * H)) * 0.05).astype(np.float16)
+    r = (g.standard_normal((1, Mp, H)) + 0.75).astype(np.float16)   # rows with a mean away from zero
+    ta, two, tw1, tw2, twq = dev(a), dev(wo), dev(w1), dev(w2), dev(wq)
+    x = dev(r)                                                      # residual stream, updated in place
+    f = torch.zeros((1, Mp, F), dtype=torch.float16, device="cuda")
+    q = torch.zeros((1, Mp, 3 * H), dtype=torch.float16, device="cuda")
+    cs1 = torch.zeros(F, dtype=torch.float32, device="cuda")
+    csq = torch.zeros(3 * H, dtype=torch.float32, device="cuda")
+    gpu.homColumnSumsF16(*M(tw1).args(), cs1.data_ptr())
+    gpu.homColumnSumsF16(*M(twq).args(), csq.data_ptr())
+    assert_close(cs1.cpu().numpy(), w1[0].astype(np.float64).sum(0), rtol=1e-5, atol=1e-4, what="column sums")
+    pieces = gpu.homFoldedLayernormPieces(Mp, H, H, 0, num)
+    assert pieces == gpu.homFoldedLayernormPieces(Mp, H, F, 0, num) or tile is None
+    st1 = torch.full((pieces * Mp * 2,), float("nan"), dtype=torch.float32, device="cuda")
+
+    def ln(v16):
+        v = v16.astype(np.float64)
+        mu = v.mean(-1, keepdims=True)
+        return (v - mu) / np.sqrt(((v - mu) ** 2).mean(-1, keepdims=True) + eps)
+
+    # x1 = a . Wo + r, in place over r, with the partial sums of x1
+    gpu.homGemmFoldedLayernormF16(*M(ta).args(), *M(two).args(), *M(x).args(), *M(x).args(), 2, 0, 1.0, 1.0,
+                                  None, 0, eps, None, st1.data_ptr(), num)
+    x1 = host(x)[0]
+    assert_close(x1, oracle.gemm(a[0], wo[0], r[0], beta=1.0), **GEMM_TOL, what="x1")
+    part = st1.cpu().numpy().reshape(pieces, Mp, 2).astype(np.float64).sum(0)
+    assert_close(part[:, 0], x1.astype(np.float64).sum(-1), rtol=1e-4, atol=1e-2, what="row sums")
+    assert_close(part[:, 1], (x1.astype(np.float64) ** 2).sum(-1), rtol=1e-4, atol=1e-2, what="row sums of squares")
+    # f = GELU(LN(x1) . W1)
+    gpu.homGemmFoldedLayernormF16(*M(x).args(), *M(tw1).args(), *M(f).args(), *M(f).args(), 1, 1, 1.0, 0.0,
+                                  st1.data_ptr(), pieces, eps, cs1.data_ptr(), None, num)
+    f16 = host(f)[0]
+    assert_close(f16, oracle.gelu(ln(x1) @ w1[0].astype(np.float64), "erf"), **GEMM_TOL, what="f")
+    # x2 = f . W2 + LN(x1), in place over x1, with the partial sums of x2
+    pieces2 = gpu.homFoldedLayernormPieces(Mp, H, F, 0, num)
+    st2 = torch.full((pieces2 * Mp * 2,), float("nan"), dtype=torch.float32, device="cuda")
+    gpu.homGemmFoldedLayernormF16(*M(f).args(), *M(tw2).args(), *M(x).args(), *M(x).args(), 2, 0, 1.0, 1.0,
+                                  st1.data_ptr(), pieces, eps, None, st2.data_ptr(), num)
+    x2 = host(x)[0]
+    assert_close(x2, f16.astype(np.float64) @ w2[0].astype(np.float64) + ln(x1), **GEMM_TOL, what="x2")
+    # q = LN(x2) . Wq
+    gpu.homGemmFoldedLayernormF16(*M(x).args(), *M(twq).args(), *M(q).args(), *M(q).args(), 1, 0, 1.0, 0.0,
+                                  st2.data_ptr(), pieces2, eps, csq.data_ptr(), None, num)
+    assert_close(host(q)[0], ln(x2) @ wq[0].astype(np.float64), **GEMM_TOL, what="q")
+    # without statistics the same entry point is the plain product
+    gpu.homGemmFoldedLayernormF16(*M(x).args(), *M(twq).args(), *M(q).args(), *M(q).args(), 1, 0, 1.0, 0.0,
+                                  None, 0, eps, None, None, num)
+    assert_close(host(q)[0], oracle.gemm(x2, wq[0]), **GEMM_TOL, what="plain product")
+
+
 # --------------------------------------------------------------- attention --
 def run_attention(gpu, rt, qkv, lens, heads, scale):
     M = rt.MemRef.from_tensor
