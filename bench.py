@@ -99,6 +99,8 @@ def main():
                          "first tens of milliseconds of launches run slower than the steady state)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-large", action="store_true", help="skip the BERT-large b32 x s512 encoder timing")
+    ap.add_argument("--no-folded", action="store_true",
+                    help="skip the optional folded-layer-norm call lists (reported beside the headline)")
     ap.add_argument("--eager", action="store_true", help="launch every call instead of replaying a HIP graph")
     ap.add_argument("--gemm-mode", type=int, default=1,
                     help="0 nvteGemmF16 path, 1 cutlassGemmF16 + tuned table, 2 + live autotune")
@@ -244,7 +246,7 @@ def main():
                                                   "TFLOP/s": big_flops / (big_ms * 1e-3) / 1e12}
         # the optional call list with the per-layer layer norms folded into the GEMMs around them
         # (5 launches per layer instead of 7; not the reference's call list, reported beside it)
-        if args.gemm_mode != 0:
+        if args.gemm_mode != 0 and not args.no_folded:
             enc = bert.BertEncoder(24, 1024, 16, 4096, 32, 512, big["dims"]["vocab"],
                                    gemm_mode=args.gemm_mode, gelu_form="erf", fold_layernorm=True)
             enc.load(big)
@@ -257,7 +259,7 @@ def main():
         del big
 
     # BERT-base through the optional folded-layer-norm call list (see above)
-    if args.gemm_mode != 0:
+    if args.gemm_mode != 0 and not args.no_folded:
         enc = bert.BertEncoder(d["layers"], d["hidden"], d["heads"], d["ffn"], d["bs"], d["seq"], d["vocab"],
                                gemm_mode=args.gemm_mode, gelu_form="erf", fold_layernorm=True)
         enc.load(model)

@@ -8,7 +8,12 @@ tile (GEMM workloads only): run the manifest kernel whose name holds `_<tile>_`
 what:  gemm1      FFN1 GEMM + bias + tanh-GELU, M=1024 K=768 N=3072 (tuned kernel)
        gemm5      BERT-large FFN2 GEMM, M=16384 K=4096 N=1024
        gemm5g     BERT-large FFN1 GEMM + bias + erf-GELU, M=16384 K=1024 N=4096
-       layernorm  in-place layer norm, 16384 x 1024
+       layernorm  in-place layer norm, 16384 x 1024, the same tensor launch after
+                  launch (it stays in the 256 MB Infinity Cache: a cache rate)
+       layernorm_cold  the same over 24 tensors walked round-robin (805 MB:
+                  every launch reads from and writes to HBM)
+       add_cold   elementwise add 16384 x 1024 over 8 (a, b, out) triples
+                  walked round-robin (805 MB)
        attention  packed-QKV attention, b8 s128 h12
        attention5 packed-QKV attention, b32 s512 h16, full-length sequences
        lnpair     the layer-norm pair at BERT-large size: GEMM + row statistics
@@ -57,6 +62,12 @@ def main():
         print(f"gemm5g {lib.homGemmManifestName(idx.value).decode()} splitK {sk.value}: {ms * 1e3:.2f} us")
     elif what == "layernorm":
         print(f"layernorm 16384x1024: {drv.homTimeLayernorm(16384, 1024, 0, iters, 3) * 1e3:.2f} us")
+    elif what == "layernorm_cold":
+        ms = drv.homTimeLayernormRotating(16384, 1024, 0, 24, iters, 3)
+        print(f"layernorm 16384x1024 over 24 rotating tensors: {ms * 1e3:.2f} us")
+    elif what == "add_cold":
+        ms = drv.homTimeElementwiseAddRotating(16384, 1024, 8, iters, 3)
+        print(f"add 16384x1024 over 8 rotating triples: {ms * 1e3:.2f} us")
     elif what == "attention":
         lens = (ctypes.c_int32 * 8)(83, 128, 57, 101, 32, 120, 64, 99)
         print(f"attention b8 s128 h12: {drv.homTimeAttention(8, 128, 12, lens, iters, 3) * 1e3:.2f} us")
