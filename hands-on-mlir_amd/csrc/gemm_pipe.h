@@ -364,6 +364,9 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(
     if constexpr (U < MI && kHandReads) {
       // (see the B units below: in this mode every fragment read is issued
       // and waited for by hand, so that the waits can be exact)
+      // INVARIANT: the registers an asm read writes are not valid until
+      // tieFragments() has waited for them; nothing may use or copy fa / fbHalf
+      // between the read and that call (the compiler believes they are ready).
       const uint32_t at = uint32_t(uintptr_t(HOM_LDS_PTR(st + aFrag[kk])));
       half8 frag;
       asm volatile("ds_read_b128 %0, %1 offset:%2"
