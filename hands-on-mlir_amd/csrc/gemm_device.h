@@ -401,7 +401,19 @@ epilogueStoreLds(const GemmParams &p, float16v (&acc)[MI][NI], int m0, int n0,
         }
         if (vec16) {
           storeWriteThrough(reinterpret_cast<half8 *>(dPtr), o);
+        } else if (n + 8 <= p.N) {
+          // rows start at 4-byte boundaries only (N even, not a multiple of 8):
+          // still one 16-byte store, which the hardware takes at dword
+          // alignment (as it does the 16-byte loads of such a B); written as
+          // asm because a C++ store of this type would promise 16-byte
+          // alignment.  Default cache policy: see store_policy.h.
+          typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+          asm volatile("global_store_dwordx4 %0, %1, off\n\ts_nop 1"
+                       :
+                       : "v"(dPtr), "v"(__builtin_bit_cast(u32x4, o))
+                       : "memory");
         } else {
+          // the row's last vector: pairs, the pair past column N is dropped
 #pragma unroll
           for (int e = 0; e < 8; e += 2)
             if (n + e < p.N) {
