@@ -285,61 +285,89 @@ __attribute__((amdgpu_waves_per_eu(D == 64 ? 2 : 1, D == 64 && KS == 1 ? 4 : 2))
       // ---- S^T = K Q^T for two 32-key sub-blocks ----
       // All eight K fragments are requested before the first MFMA: read one
       // at a time, each MFMA would wait out a full LDS round trip.
-      half8 fk[2][kHeadDim / 16];
-#pragma unroll
-      for (int sb = 0; sb < 2; sb++)
-#pragma unroll
-        for (int kk = 0; kk < kHeadDim / 16; kk++)
-          fk[sb][kk] = *reinterpret_cast<const half8 *>(
-              sK + (blk + sb * 32 + l32) * kRowB + ((kk * 2 + hb) ^ swzLane) * 16);
-      __builtin_amdgcn_sched_barrier(0);
-      float16v accS[2];
-#pragma unroll
-      for (int sb = 0; sb < 2; sb++) {
-#pragma unroll
-        for (int e = 0; e < 16; e++)
-          accS[sb][e] = 0.f;
-#pragma unroll
-        for (int kk = 0; kk < kHeadDim / 16; kk++)
-          accS[sb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fk[sb][kk], fq[kk],
-                                                            accS[sb], 0, 0, 0);
-      }
       // accS[sb][e] is the raw score (before scaling) of query l32 against key
       //   key0 + blk + sb*32 + 8*(e/4) + 4*hb + e%4.
+      // Only a block that reaches past the sequence end pays for the key mask.
+      float16v accS[2];
+      auto scores = [&]() {
+        half8 fk[2][kHeadDim / 16];
+#pragma unroll
+        for (int sb = 0; sb < 2; sb++)
+#pragma unroll
+          for (int kk = 0; kk < kHeadDim / 16; kk++)
+            fk[sb][kk] = *reinterpret_cast<const half8 *>(
+                sK + (blk + sb * 32 + l32) * kRowB + ((kk * 2 + hb) ^ swzLane) * 16);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int sb = 0; sb < 2; sb++) {
+#pragma unroll
+          for (int e = 0; e < 16; e++)
+            accS[sb][e] = 0.f;
+#pragma unroll
+          for (int kk = 0; kk < kHeadDim / 16; kk++)
+            accS[sb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fk[sb][kk], fq[kk],
+                                                              accS[sb], 0, 0, 0);
+        }
+        if (key0 + blk + 64 > len) {
+#pragma unroll
+          for (int sb = 0; sb < 2; sb++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) {
+              const int key = key0 + blk + sb * 32 + 8 * (e / 4) + 4 * hb + (e % 4);
+              accS[sb][e] = key < len ? accS[sb][e] : -INFINITY;
+            }
+        }
+      };
+      scores();
       // The softmax works on raw scores: with c = scale * log2(e) > 0,
       // exp(scale * (s - m)) = exp2(c * s - c * m), one FMA and one v_exp per
-      // score; the running maximum is kept in raw units.  Only a block that
-      // reaches past the sequence end pays for the key mask.  This part is
-      // VALU work the matrix core cannot hide (16 MFMAs against several
-      // hundred vector instructions per block), so instruction count matters.
-      if (key0 + blk + 64 > len) {
+      // score; the reference m (rowMax, raw units) only has to keep p within
+      // range, it need not be the true maximum, and the final O / rowSum cancels
+      // whatever reference was used.  This part is VALU work the matrix core
+      // cannot hide (16 MFMAs against a few hundred vector instructions per
+      // block), so instruction count matters:
+      //  - fast path (every block but a wavefront's first): p is computed
+      //    against the reference as it stands, no maximum is taken at all, and
+      //    the row sums that are needed anyway tell whether that was safe: if
+      //    some row's sum over the 64 keys exceeds kSumLimit (so a p could leave
+      //    fp16's range; an overflowed exp2 gives inf and lands here too) the
+      //    block's scores are recomputed from LDS and take the slow path;
+      //  - slow path (the first block, and a block whose sums overflowed): the
+      //    true block maximum, the reference moves to it, O and the running
+      //    sum are rescaled (96 vector instructions on the accumulators).
+      // With real score distributions the slow path runs once per wavefront.
+      // Every block that is visited has at least one valid key, so blockMax
+      // is finite and the differences below are never inf - inf.
+      constexpr float kSumLimit = 4096.0f;
+      const bool first = ch == 0 && blk == kh * 64;
+      float blockSum = 0.f;
+      bool slow = first;
+      if (!first) {
+        const float negMax = -rowMax * scaleLog2e;
 #pragma unroll
         for (int sb = 0; sb < 2; sb++)
 #pragma unroll
           for (int e = 0; e < 16; e++) {
-            const int key = key0 + blk + sb * 32 + 8 * (e / 4) + 4 * hb + (e % 4);
-            accS[sb][e] = key < len ? accS[sb][e] : -INFINITY;
+            const float pv =
+                __builtin_amdgcn_exp2f(fmaf(accS[sb][e], scaleLog2e, negMax));
+            accS[sb][e] = pv;
+            blockSum += pv;
           }
+        blockSum = pairSum(blockSum);
+        slow = __any(!(blockSum <= kSumLimit));
+        if (slow)
+          scores(); // the probabilities are discarded: raw scores again
       }
-      float blockMax = -INFINITY;
+      if (slow) {
+        float blockMax = -INFINITY;
 #pragma unroll
-      for (int sb = 0; sb < 2; sb++)
+        for (int sb = 0; sb < 2; sb++)
 #pragma unroll
-        for (int e = 0; e < 16; e++)
-          blockMax = fmaxf(blockMax, accS[sb][e]);
-      blockMax = pairMax(blockMax);
-      // The exponent's reference rowMax only has to keep p within range, it
-      // need not be the true maximum: it moves (and O and the running sum are
-      // rescaled, 96 vector instructions on the accumulators) only when some
-      // row of the wavefront has grown past it by more than kSlack in the
-      // exponent, i.e. p would exceed 2^kSlack.  The final O / rowSum cancels
-      // whatever reference was used.  With real score distributions that
-      // happens in the first block or two of a row and rarely afterwards.
-      // Every block that is visited has at least one valid key, so blockMax
-      // is finite and the differences below are never inf - inf.
-      constexpr float kSlack = 8.0f;
-      if (__any((blockMax - rowMax) * scaleLog2e > kSlack)) {
+          for (int e = 0; e < 16; e++)
+            blockMax = fmaxf(blockMax, accS[sb][e]);
+        blockMax = pairMax(blockMax);
         const float newMax = fmaxf(rowMax, blockMax);
+        // (first block: rowMax = -inf, corr = 0 on accumulators that are 0)
         const float corr = __builtin_amdgcn_exp2f((rowMax - newMax) * scaleLog2e);
         rowSum *= corr;
         rowMax = newMax;
@@ -348,19 +376,19 @@ __attribute__((amdgpu_waves_per_eu(D == 64 ? 2 : 1, D == 64 && KS == 1 ? 4 : 2))
 #pragma unroll
           for (int e = 0; e < 16; e++)
             accO[d][e] *= corr;
+        const float negMax = -rowMax * scaleLog2e;
+        blockSum = 0.f;
+#pragma unroll
+        for (int sb = 0; sb < 2; sb++)
+#pragma unroll
+          for (int e = 0; e < 16; e++) {
+            const float pv =
+                __builtin_amdgcn_exp2f(fmaf(accS[sb][e], scaleLog2e, negMax));
+            accS[sb][e] = pv;
+            blockSum += pv;
+          }
+        blockSum = pairSum(blockSum);
       }
-      const float negMax = -rowMax * scaleLog2e;
-      float blockSum = 0.f;
-#pragma unroll
-      for (int sb = 0; sb < 2; sb++)
-#pragma unroll
-        for (int e = 0; e < 16; e++) {
-          const float pv =
-              __builtin_amdgcn_exp2f(fmaf(accS[sb][e], scaleLog2e, negMax));
-          accS[sb][e] = pv;
-          blockSum += pv;
-        }
-      blockSum = pairSum(blockSum);
       rowSum += blockSum;
 
       // ---- O^T += V^T P^T ----

@@ -610,6 +610,26 @@ def test_attention_head_size_128(gpu, rt, oracle, bs, seq, heads, lens):
     assert np.array_equal(one.reshape(1, 64, heads, 128), want)
 
 
+@pytest.mark.parametrize("d,heads", [(64, 4), (128, 2)])
+def test_attention_growing_scores(gpu, rt, oracle, d, heads):
+    """Scores that keep growing along the keys: the softmax reference a wavefront fixed on its first key block
+    has to move again and again (the probabilities of a later block would leave fp16's range against the old
+    reference), in blocks of any position, with full and ragged lengths, in both kernel variants."""
+    g = np.random.default_rng(d + heads)
+    for bs, seq, lens in ((2, 512, [512, 301]), (32, 512, None), (3, 128, [128, 70, 9])):
+        qkv = g.standard_normal((bs, seq, 3, heads, d)).astype(np.float32)
+        ramp = 1.0 + 5.0 * np.arange(seq, dtype=np.float32) / seq        # keys 6 times larger at the end
+        qkv[:, :, 1] *= ramp[None, :, None, None]
+        qkv[:, seq // 2, 1] *= 2.0                                         # and a spike in the middle
+        qkv = qkv.reshape(bs, seq, -1).astype(np.float16)
+        lens_ = np.array(lens if lens is not None else g.integers(1, seq + 1, size=bs), np.int32)
+        scale = 1.0 / np.sqrt(float(d))
+        got, cu = run_attention(gpu, rt, qkv, lens_, heads, scale)
+        assert np.isfinite(got.astype(np.float32)).all()
+        assert_close(got, oracle.attention(qkv, cu, heads, scale), **GEMM_TOL,
+                     what=f"attention d{d} {bs}x{seq}, growing scores")
+
+
 def test_attention_layout_onehot(gpu, rt):
     """Pins the [3][heads][64] interleave: V one-hot in (head 5, d 9)."""
     heads, seq = 12, 64
