@@ -9,6 +9,7 @@
 //   row stats    include/NVGPUKernels/Layernorm.h:33-195 (ApplyFinalReduction)
 #include "cross_lane.h"
 #include "kernels.h"
+#include "store_policy.h"
 
 namespace hom {
 namespace {

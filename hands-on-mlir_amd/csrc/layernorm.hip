@@ -37,8 +37,11 @@ template <> struct Vec16<float> {
 // and written with the non-temporal hint, because nothing is touched twice and
 // without the hint the written rows linger in the L2s and compete with the
 // reads on their way out (16384 x 1024 in place, rotating over 800 MB so that
-// every launch is cold: 4.5 TB/s with default accesses, 5.4 TB/s with the hint;
-// a plain read-modify-write probe shows the same 4.7 -> 5.65 TB/s).
+// every launch is cold: 4.5 TB/s with default accesses, 5.4 TB/s with the hint,
+// 5.6 TB/s with the in-place form's stores also written through; a plain
+// read-modify-write probe shows the same 4.65 -> 5.55 -> 5.72 TB/s.  With a
+// residual operand, two read streams and a write stream, writing through costs
+// 1 % instead: 17.4 against 17.5 us).
 //
 // The kernel is a chain of memory round trips (arguments, row, result) a few
 // hundred nanoseconds each, so everything it will read is requested at once and
@@ -132,7 +135,9 @@ __global__ __launch_bounds__(256) void layernormWaveKernel(
       o[j] = T(y);
     }
     if (rowOk && idx < nvec) {
-      if (STREAM)
+      if (STREAM && !HAS_RES)
+        storeStreaming(&orow[idx], o); // the in-place form: see store_policy.h
+      else if (STREAM)
         __builtin_nontemporal_store(o, &orow[idx]);
       else
         storeWriteThrough(&orow[idx], o);

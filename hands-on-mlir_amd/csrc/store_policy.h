@@ -59,4 +59,21 @@ __device__ __forceinline__ void storeWriteThrough(V *p, const V &v) {
   }
 }
 
+// *p = v for 16-byte results of kernels that stream tensors larger than the
+// last-level cache (nothing is read again soon): written through and marked
+// non-temporal.  A cold in-place read-modify-write stream of 33.5 MB measured
+// 4.65 TB/s with default accesses, 5.55 TB/s with the non-temporal hint on
+// loads and stores, 5.72 TB/s with this store policy on top (sc1 nt; sc0 sc1
+// nt is the same); write-through without the hint 5.49 TB/s.
+template <typename V>
+__device__ __forceinline__ void storeStreaming(V *p, const V &v) {
+  static_assert(sizeof(V) == 16, "store width");
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+  // (wait states: see storeWriteThrough)
+  asm volatile("global_store_dwordx4 %0, %1, off sc1 nt\n\ts_nop 1"
+               :
+               : "v"(p), "v"(__builtin_bit_cast(u32x4, v))
+               : "memory");
+}
+
 } // namespace hom
