@@ -44,24 +44,35 @@ typedef short short4v __attribute__((ext_vector_type(4)));
 typedef short short8v __attribute__((ext_vector_type(8)));
 
 constexpr int kWave = 64;
-constexpr int kChunk = 128;                  // keys staged per barrier
-
-// Head sizes 64 and 128 (template parameter D).  A K or V row in LDS is D
-// halves: 128 bytes = 8 chunks of 16 bytes = 2 groups of 64 bytes for D = 64,
-// twice that for D = 128.
+// Head sizes 64, 128, 192 and 256 (template parameter D; the reference's
+// contract is head size % 64 == 0).  64 is what every BERT configuration has
+// and what the kernel is tuned for, 128 is the same code with twice the
+// registers, 192 and 256 are functional (one wavefront per SIMD, half the keys
+// per LDS chunk, staging addresses computed per vector).  A K or V row in LDS
+// is D halves: 128 bytes = 8 chunks of 16 bytes = 2 groups of 64 bytes for
+// D = 64.
 //
+// Keys staged per barrier: 128, or 64 where two tiles of 128 rows would not fit
+// the 64 KB of static LDS.
+template <int D> struct Chunk {
+  static constexpr int value = D <= 128 ? 128 : 64;
+};
 // chunk c (16 bytes) of K row r lives at position c ^ ((r >> 1) & 7) (rows of
 // 128 bytes: two consecutive rows cover all banks once) or c ^ (r & 15) (rows
-// of 256 bytes: every row starts at bank 0), so that the 128-bit fragment
-// reads of 16 consecutive rows hit 16 distinct bank groups
+// of 256 or 512 bytes: every row starts at bank 0), so that the 128-bit
+// fragment reads of 16 consecutive rows hit 16 distinct bank groups; rows of
+// 384 bytes (24 chunks) permute inside groups of 8 chunks so that a position
+// never leaves the row
 template <int D> __device__ __forceinline__ int swzK(int row, int chunk) {
-  return D == 64 ? chunk ^ ((row >> 1) & 7) : chunk ^ (row & 15);
+  return D == 64    ? chunk ^ ((row >> 1) & 7)
+         : D == 192 ? chunk ^ (row & 7)
+                    : chunk ^ (row & 15);
 }
 // 64-byte group g of V row k lives at position g ^ ((k >> 1) & 1), or
-// g ^ (k & 3) for rows of 256 bytes: a transposing read touches 64 bytes of
-// each of rows k..k+3
+// g ^ (k & 3) for rows whose group count is a multiple of 4: a transposing read
+// touches 64 bytes of each of rows k..k+3
 template <int D> __device__ __forceinline__ int swzV(int k, int group) {
-  return D == 64 ? group ^ ((k >> 1) & 1) : group ^ (k & 3);
+  return D == 64 || D == 192 ? group ^ ((k >> 1) & 1) : group ^ (k & 3);
 }
 
 // NW wavefronts per workgroup, KS of them share each group of 32 query rows
@@ -71,11 +82,13 @@ template <int D> __device__ __forceinline__ int swzV(int k, int group) {
 // of one wavefront is the critical path; the halves are merged through LDS).
 template <int NW, int KS, int D>
 __global__ __launch_bounds__(NW *kWave)
-__attribute__((amdgpu_waves_per_eu(D == 64 ? 2 : 1, D == 64 && KS == 1 ? 4 : 2))) void bertAttentionKernel(
+__attribute__((amdgpu_waves_per_eu(D == 64 ? 2 : 1, D == 64 && KS == 1 ? 4 : (D <= 128 ? 2 : 1)))) void bertAttentionKernel(
     const _Float16 *__restrict__ qkv, const int32_t *__restrict__ cu,
     _Float16 *__restrict__ out, int seq, int heads, int numQTiles, int pairs,
     float scale) {
-  static_assert(D == 64 || D == 128, "head size");
+  static_assert(D == 64 || D == 128 || D == 192 || D == 256, "head size");
+  static_assert(D <= 128 || KS == 1, "the key-split variant stages 128 keys per chunk");
+  constexpr int kChunk = Chunk<D>::value;
   constexpr int kHeadDim = D;
   constexpr int kRowB = D * 2;               // bytes of a K or V row
   constexpr int CPR = D / 8;                 // 16-byte chunks per row
@@ -212,12 +225,15 @@ __attribute__((amdgpu_waves_per_eu(D == 64 ? 2 : 1, D == 64 && KS == 1 ? 4 : 2))
   // t / 8 + i * kThreads / 8.  Both swizzles depend on row bits that the
   // per-vector row step (a multiple of 16) leaves alone, so the LDS
   // destinations are one base plus immediates.
+  // (Head sizes above 128: the row step is not a multiple of 16, or not a
+  // whole number; those compute every vector's addresses, see below.)
+  constexpr bool kFastStage = kThreads % CPR == 0 && (kThreads / CPR) % 16 == 0;
+  static_assert(kFastStage || D > 128, "row step per vector must leave the swizzles alone");
   const uint32_t rowBytes = uint32_t(tokStride) * 2u;
   const uint32_t stageOff = uint32_t(tid / CPR) * rowBytes + uint32_t(tid % CPR) * 16u;
   const int stageK = (tid / CPR) * kRowB + swzK<D>(tid / CPR, tid % CPR) * 16;
   const int stageV = (tid / CPR) * kRowB + swzV<D>(tid / CPR, (tid % CPR) / 4) * 64 +
                      ((tid % CPR) % 4) * 16;
-  static_assert((kThreads / CPR) % 16 == 0, "row step per vector must leave the swizzles alone");
   const auto rsrcK = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<_Float16 *>(kBase), 0, int32_t(uint32_t(len) * rowBytes),
       0x00020000);
@@ -262,19 +278,42 @@ __attribute__((amdgpu_waves_per_eu(D == 64 ? 2 : 1, D == 64 && KS == 1 ? 4 : 2))
       // past the sequence read as zero without touching memory.  All loads go
       // out before the first LDS store; addresses are one add per vector.
       half8 kv[VPT], vv[VPT];
-      const uint32_t chunkOff = stageOff + uint32_t(key0) * rowBytes;
+      if constexpr (kFastStage) {
+        const uint32_t chunkOff = stageOff + uint32_t(key0) * rowBytes;
 #pragma unroll
-      for (int i = 0; i < VPT; i++) {
-        const uint32_t off = chunkOff + uint32_t(i * (kThreads / CPR)) * rowBytes;
-        kv[i] = __builtin_bit_cast(
-            half8, __builtin_amdgcn_raw_buffer_load_b128(rsrcK, off, 0, 0));
-        vv[i] = __builtin_bit_cast(
-            half8, __builtin_amdgcn_raw_buffer_load_b128(rsrcV, off, 0, 0));
-      }
+        for (int i = 0; i < VPT; i++) {
+          const uint32_t off = chunkOff + uint32_t(i * (kThreads / CPR)) * rowBytes;
+          kv[i] = __builtin_bit_cast(
+              half8, __builtin_amdgcn_raw_buffer_load_b128(rsrcK, off, 0, 0));
+          vv[i] = __builtin_bit_cast(
+              half8, __builtin_amdgcn_raw_buffer_load_b128(rsrcV, off, 0, 0));
+        }
 #pragma unroll
-      for (int i = 0; i < VPT; i++) {
-        *reinterpret_cast<half8 *>(sK + stageK + i * (kThreads / CPR) * kRowB) = kv[i];
-        *reinterpret_cast<half8 *>(sV + stageV + i * (kThreads / CPR) * kRowB) = vv[i];
+        for (int i = 0; i < VPT; i++) {
+          *reinterpret_cast<half8 *>(sK + stageK + i * (kThreads / CPR) * kRowB) = kv[i];
+          *reinterpret_cast<half8 *>(sV + stageV + i * (kThreads / CPR) * kRowB) = vv[i];
+        }
+      } else {
+        // vector v of the chunk = 16-byte chunk v % CPR of row v / CPR
+        static_assert((kChunk * CPR) % kThreads == 0, "whole vectors per thread");
+#pragma unroll
+        for (int i = 0; i < VPT; i++) {
+          const int v = tid + i * kThreads;
+          const uint32_t off =
+              uint32_t(key0 + v / CPR) * rowBytes + uint32_t(v % CPR) * 16u;
+          kv[i] = __builtin_bit_cast(
+              half8, __builtin_amdgcn_raw_buffer_load_b128(rsrcK, off, 0, 0));
+          vv[i] = __builtin_bit_cast(
+              half8, __builtin_amdgcn_raw_buffer_load_b128(rsrcV, off, 0, 0));
+        }
+#pragma unroll
+        for (int i = 0; i < VPT; i++) {
+          const int v = tid + i * kThreads;
+          const int r = v / CPR, c = v % CPR;
+          *reinterpret_cast<half8 *>(sK + r * kRowB + swzK<D>(r, c) * 16) = kv[i];
+          *reinterpret_cast<half8 *>(sV + r * kRowB + swzV<D>(r, c / 4) * 64 +
+                                     (c % 4) * 16) = vv[i];
+        }
       }
     }
     if (kPrefetch && ch + 1 < numChunks)
@@ -491,9 +530,10 @@ Status launchBertAttentionF16(const _Float16 *qkv, const int32_t *cuSeqlens,
                               int64_t heads, int64_t headDim, float scale,
                               hipStream_t s) {
   // (the reference's contract is head size % 64 == 0, README.md:11; the
-  // sizes with kernels here are 64 and 128)
-  HOM_CHECK_RET(headDim == 64 || headDim == 128, Status::kInvalidArgument,
-                "attention: head size %lld not supported (64 or 128)",
+  // sizes with kernels here are 64, 128, 192 and 256)
+  HOM_CHECK_RET(headDim == 64 || headDim == 128 || headDim == 192 || headDim == 256,
+                Status::kInvalidArgument,
+                "attention: head size %lld not supported (64, 128, 192 or 256)",
                 (long long)headDim);
   // The softmax tracks the maximum of the unscaled scores, which is the
   // maximum of the scaled ones only for a positive scale (BERT: 1/sqrt(64)).
@@ -519,6 +559,8 @@ Status launchBertAttentionF16(const _Float16 *qkv, const int32_t *cuSeqlens,
   // profiling knob: HOM_ATTENTION_VARIANT=wide | split
   if (const char *force = getenv("HOM_ATTENTION_VARIANT"))
     wide = strcmp(force, "wide") == 0;
+  if (headDim > 128)
+    wide = true; // (the key-split variant exists for 64 and 128 only)
   HOM_CHECK_RET(pairs * ((seq + 63) / 64) < (int64_t(1) << 31),
                 Status::kInvalidArgument, "attention: too many workgroups");
   if (wide) {
@@ -527,8 +569,14 @@ Status launchBertAttentionF16(const _Float16 *qkv, const int32_t *cuSeqlens,
     if (headDim == 64)
       bertAttentionKernel<4, 1, 64><<<grid, dim3(256), 0, s>>>(
           qkv, cuSeqlens, out, int(seq), int(heads), nq, int(pairs), scale);
-    else
+    else if (headDim == 128)
       bertAttentionKernel<4, 1, 128><<<grid, dim3(256), 0, s>>>(
+          qkv, cuSeqlens, out, int(seq), int(heads), nq, int(pairs), scale);
+    else if (headDim == 192)
+      bertAttentionKernel<4, 1, 192><<<grid, dim3(256), 0, s>>>(
+          qkv, cuSeqlens, out, int(seq), int(heads), nq, int(pairs), scale);
+    else
+      bertAttentionKernel<4, 1, 256><<<grid, dim3(256), 0, s>>>(
           qkv, cuSeqlens, out, int(seq), int(heads), nq, int(pairs), scale);
   } else {
     const int nq = int((seq + 63) / 64);

@@ -52,7 +52,7 @@ Status launchApplyRowStatsF16(const _Float16 *a, const _Float16 *var,
 
 // ------------------------------------------------------------- attention --
 // qkv [bs, seq, 3*heads*headDim] fp16, cu int32[bs+1], out [bs, seq,
-// heads*headDim].  headDim must be 64.
+// heads*headDim].  headDim 64, 128, 192 or 256.
 Status launchBertAttentionF16(const _Float16 *qkv, const int32_t *cuSeqlens,
                               _Float16 *out, int64_t bs, int64_t seq,
                               int64_t heads, int64_t headDim, float scale,

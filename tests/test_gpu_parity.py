@@ -586,31 +586,48 @@ def test_attention_shapes_and_edges(gpu, rt, oracle, bs, seq, heads, lens):
     assert_close(got, oracle.attention(qkv, cu, heads, 0.125), **GEMM_TOL, what=f"attention {bs}x{seq}x{heads}")
 
 
+@pytest.mark.parametrize("d", [128, 192, 256])
 @pytest.mark.parametrize("bs,seq,heads,lens", [
     (2, 64, 2, [64, 1]), (3, 100, 1, [100, 37, 64]), (2, 512, 8, [512, 300]),
     (4, 128, 6, [0, 128, 65, 33]), (1, 40, 3, [17]), (16, 512, 4, None)])
-def test_attention_head_size_128(gpu, rt, oracle, bs, seq, heads, lens):
-    """Head size 128 (the reference's contract is head size % 64 == 0): both kernel variants (the
-    larger shapes take 128 query rows per workgroup, the smaller ones the key-split form), padding,
-    an empty sequence, ragged lengths; padded query rows are zeros."""
-    g = np.random.default_rng(bs * 1000 + seq + 7)
-    qkv = g.standard_normal((bs, seq, 3 * heads * 128)).astype(np.float16)
+def test_attention_larger_head_sizes(gpu, rt, oracle, d, bs, seq, heads, lens):
+    """Head sizes 128, 192 and 256 (the reference's contract is head size % 64 == 0): both kernel variants
+    where they exist (d = 128: the larger shapes take 128 query rows per workgroup, the smaller ones the
+    key-split form), padding, an empty sequence, ragged lengths; padded query rows are zeros."""
+    g = np.random.default_rng(bs * 1000 + seq + 7 + d)
+    qkv = g.standard_normal((bs, seq, 3 * heads * d)).astype(np.float16)
     lens = np.array(lens if lens is not None else g.integers(1, seq + 1, size=bs), np.int32)
-    scale = 1.0 / np.sqrt(128.0)
+    scale = 1.0 / np.sqrt(float(d))
     got, cu = run_attention(gpu, rt, qkv, lens, heads, scale)
-    assert_close(got, oracle.attention(qkv, cu, heads, scale), **GEMM_TOL, what=f"attention d128 {bs}x{seq}x{heads}")
+    assert_close(got, oracle.attention(qkv, cu, heads, scale), **GEMM_TOL, what=f"attention d{d} {bs}x{seq}x{heads}")
     for b, n in enumerate(lens):
         assert not got[b, n:].any(), "padded query rows must be zeros"
-    # layout: V one-hot in (head h, column 77) comes out in (head h, column 77) of every valid row
-    z = np.zeros((1, 64, 3, heads, 128), np.float16)
-    z[:, :, 2, heads - 1, 77] = 1.0
+    # layout: V one-hot in (head h, column d - 51) comes out in that column of every valid row
+    col = d - 51
+    z = np.zeros((1, 64, 3, heads, d), np.float16)
+    z[:, :, 2, heads - 1, col] = 1.0
     one, _ = run_attention(gpu, rt, z.reshape(1, 64, -1), [64], heads, scale)
-    want = np.zeros((1, 64, heads, 128), np.float16)
-    want[:, :, heads - 1, 77] = 1.0
-    assert np.array_equal(one.reshape(1, 64, heads, 128), want)
+    want = np.zeros((1, 64, heads, d), np.float16)
+    want[:, :, heads - 1, col] = 1.0
+    assert np.array_equal(one.reshape(1, 64, heads, d), want)
 
 
-@pytest.mark.parametrize("d,heads", [(64, 4), (128, 2)])
+def test_attention_rejects_other_head_sizes(gpu, rt):
+    M = rt.MemRef.from_tensor
+    qkv = torch.zeros((1, 64, 3 * 2 * 96), dtype=torch.float16, device="cuda")
+    cu = torch.tensor([0, 64], dtype=torch.int32, device="cuda")
+    out = torch.zeros((1, 64, 2 * 96), dtype=torch.float16, device="cuda")
+    gpu.homSetErrorMode(1)
+    try:
+        gpu.homGetLastError()
+        gpu.nvteBertAttentionF16(*M(qkv).args(), *M(cu).args(), *M(out).args(), 0.1, 2)
+        msg = gpu.homGetLastError().decode()
+    finally:
+        gpu.homSetErrorMode(0)
+    assert "head size" in msg, msg
+
+
+@pytest.mark.parametrize("d,heads", [(64, 4), (128, 2), (256, 1)])
 def test_attention_growing_scores(gpu, rt, oracle, d, heads):
     """Scores that keep growing along the keys: the softmax reference a wavefront fixed on its first key block
     has to move again and again (the probabilities of a later block would leave fp16's range against the old
