@@ -259,3 +259,26 @@ def test_binary_constant_files(rt, tmp_path, monkeypatch):
     assert "not a HOMW v1 rank-3 file" in _errors(rt, lambda lib: lib.allocConstantNVGPUF16(3))
     assert "holds 23 values, expected 24" in _errors(rt, lambda lib: lib.allocConstantNVGPUF16(4))
 
+
+
+def test_folded_layernorm_gemm_argument_checks(rt):
+    """The folded layer norm + GEMM entry point refuses what its kernels do not implement, before any launch."""
+    M = rt.MemRef
+    a, b, d = M(256, [1, 64, 128]), M(256, [1, 128, 64]), M(256, [1, 64, 64])
+    stats = ctypes.c_void_p(4096)
+
+    def call(mode, act=0, beta=0.0, stats_in=None, col=None, stats_out=None, pieces=1, A=a, B=b):
+        return lambda lib: lib.homGemmFoldedLayernormF16(*A.args(), *B.args(), *d.args(), *d.args(), mode, act, 1.0,
+                                                         beta, stats_in, pieces, 1e-5, col, stats_out, 0)
+    assert "mode must be 1" in _errors(rt, call(3))
+    assert "0 pieces" in _errors(rt, call(1, stats_in=stats, col=stats, pieces=0))
+    assert "not supported" in _errors(rt, call(1, stats_in=stats))                 # normalising A needs colsum(B)
+    assert "not supported" in _errors(rt, call(1, stats_out=stats))                # mode 1 emits no sums
+    assert "not supported" in _errors(rt, call(2, act=1, beta=1.0))                # no activation after the residual
+    assert "not supported" in _errors(rt, call(2, stats_in=stats, beta=0.0))       # nothing to normalise
+    assert "K mismatch" in _errors(rt, call(1, B=M(256, [1, 120, 64])))
+    assert "column sums" in _errors(rt, lambda lib: lib.homColumnSumsF16(2, M(256, [128, 64]).descriptor, stats))
+    lib = rt.load_runtime()
+    for (m, n, k) in [(1024, 768, 768), (16384, 1024, 1024), (64, 64, 64)]:
+        pieces = lib.homFoldedLayernormPieces(m, n, k, 0, 0)
+        assert 1 <= pieces <= (n + 63) // 64 and pieces in {-(-n // e) for e in (64, 128, 256)}
