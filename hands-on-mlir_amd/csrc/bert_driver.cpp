@@ -750,20 +750,108 @@ void fillRandomF16(void *dev, int64_t numel, float scale, uint32_t seed) {
 }
 } // namespace
 
+// What the matrix cores deliver when nothing else is in the way: every
+// wavefront (two per SIMD, the occupancy of the large GEMM tiles) issues
+// v_mfma_f32_32x32x16_f16 back to back on operands that never leave its
+// registers, four independent accumulator blocks, no memory access inside the
+// loop.  VALU_PER_MFMA independent fp32 FMAs are placed behind every MFMA.
+typedef _Float16 ProbeHalf8 __attribute__((ext_vector_type(8)));
+typedef float ProbeFloat16 __attribute__((ext_vector_type(16)));
+template <int VALU_PER_MFMA>
+__global__ __launch_bounds__(512) void mfmaCeilingKernel(const _Float16 *in,
+                                                         float *out, int iters) {
+  ProbeHalf8 a, b;
+  for (int i = 0; i < 8; ++i) {
+    a[i] = in[(threadIdx.x * 8 + i) & 4095];
+    b[i] = in[4096 + ((threadIdx.x * 8 + i) & 4095)];
+  }
+  ProbeFloat16 acc[4] = {};
+  float x[8];
+  for (int i = 0; i < 8; ++i)
+    x[i] = float(in[(i + threadIdx.x) & 4095]);
+  const float c = float(in[3]) * 1e-3f + 1.0f, d = float(in[5]);
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      acc[j & 3] =
+          __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc[j & 3], 0, 0, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+#pragma unroll
+      for (int v = 0; v < VALU_PER_MFMA; ++v) {
+        const int k = (j * VALU_PER_MFMA + v) & 7;
+        x[k] = fmaf(x[k], c, d);
+      }
+      if (VALU_PER_MFMA)
+        __builtin_amdgcn_sched_group_barrier(0x002, VALU_PER_MFMA, 0);
+    }
+  }
+  float s = 0;
+  for (int i = 0; i < 8; ++i)
+    s += x[i];
+  for (int k = 0; k < 4; ++k)
+    for (int i = 0; i < 16; ++i)
+      s += acc[k][i];
+  out[blockIdx.x * 512 + threadIdx.x] = s;
+}
+
+// TFLOP/s of that loop on one workgroup of 8 wavefronts per CU.
+// randomOperands: 0 = all operands zero, 1 = values in [-1, 1).  valuPerMfma:
+// 0, 4 or 8.  Negative on error.
+DRV_EXPORT double homMfmaCeilingProbe(int randomOperands, int valuPerMfma) {
+  const int n = 8192;
+  Tensor in, out;
+  in.m = alloc3DMemRefNVGPUF16(1, 1, n);
+  out.m = alloc3DMemRefNVGPUF16(1, 512, 2 * 512); // 256 * 512 floats
+  if (!in.data() || !out.data())
+    return -1.0;
+  if (randomOperands)
+    fillRandomF16(in.data(), n, 0.5f, 11);
+  else
+    (void)hipMemset(in.data(), 0, size_t(n) * 2);
+  const int iters = 4000, launches = 5;
+  double tflops = -1.0;
+  {
+    Timer t;
+    auto call = [&] {
+      const _Float16 *src = static_cast<const _Float16 *>(in.data());
+      float *dst = static_cast<float *>(out.data());
+      if (valuPerMfma >= 8)
+        mfmaCeilingKernel<8><<<256, 512, 0, t.s>>>(src, dst, iters);
+      else if (valuPerMfma >= 4)
+        mfmaCeilingKernel<4><<<256, 512, 0, t.s>>>(src, dst, iters);
+      else
+        mfmaCeilingKernel<0><<<256, 512, 0, t.s>>>(src, dst, iters);
+    };
+    const double ms = t.run(call, launches, 2);
+    // 256 workgroups x 8 wavefronts x 16 MFMAs of 32 x 32 x 16 per iteration
+    if (ms > 0)
+      tflops = 256.0 * 8 * 16 * iters * (2.0 * 32 * 32 * 16) / (ms * 1e-3) / 1e12;
+  }
+  in.release();
+  out.release();
+  return tflops;
+}
+
 // D = act(A.B + bias) with bias broadcast as a [1,1,N] C (useBias) or beta = 0.
 // gemmNum is 1-based (0 = library picks); returns ms per call.  inGraph != 0:
 // 100 calls per captured graph, iters / 100 replays.
 static double timeGemm(int64_t M, int64_t N, int64_t K, int64_t act,
                        int useBias, int32_t gemmNum, int32_t splitK, int iters,
-                       int warmup, int inGraph) {
+                       int warmup, int inGraph, bool zeroOperands = false) {
   Tensor a, b, c, d;
   a.m = alloc3DMemRefNVGPUF16(1, int32_t(M), int32_t(K));
   b.m = alloc3DMemRefNVGPUF16(1, int32_t(K), int32_t(N));
   c.m = alloc3DMemRefNVGPUF16(1, 1, int32_t(N));
   d.m = alloc3DMemRefNVGPUF16(1, int32_t(M), int32_t(N));
-  fillRandomF16(a.data(), M * K, 1.0f, 1);
-  fillRandomF16(b.data(), K * N, 0.02f, 2);
-  fillRandomF16(c.data(), N, 0.02f, 3);
+  if (zeroOperands) {
+    (void)hipMemset(a.data(), 0, size_t(M * K) * 2);
+    (void)hipMemset(b.data(), 0, size_t(K * N) * 2);
+    (void)hipMemset(c.data(), 0, size_t(N) * 2);
+  } else {
+    fillRandomF16(a.data(), M * K, 1.0f, 1);
+    fillRandomF16(b.data(), K * N, 0.02f, 2);
+    fillRandomF16(c.data(), N, 0.02f, 3);
+  }
   double ms;
   {
     Timer t;
@@ -787,6 +875,18 @@ DRV_EXPORT double homTimeGemm(int64_t M, int64_t N, int64_t K, int64_t act,
                               int useBias, int32_t gemmNum, int32_t splitK,
                               int iters, int warmup) {
   return timeGemm(M, N, K, act, useBias, gemmNum, splitK, iters, warmup, 0);
+}
+
+// The same kernel on operands that are all zero: identical instructions and
+// memory traffic, no switching in the data paths.  What it gains over
+// homTimeGemm is what the chip's power management takes from the kernel on
+// real data.
+DRV_EXPORT double homTimeGemmZeroOperands(int64_t M, int64_t N, int64_t K,
+                                          int64_t act, int useBias,
+                                          int32_t gemmNum, int32_t splitK,
+                                          int iters, int warmup) {
+  return timeGemm(M, N, K, act, useBias, gemmNum, splitK, iters, warmup, 0,
+                  true);
 }
 
 DRV_EXPORT double homTimeGemmInGraph(int64_t M, int64_t N, int64_t K,

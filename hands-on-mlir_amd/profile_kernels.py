@@ -21,6 +21,13 @@ what:  gemm1      FFN1 GEMM + bias + tanh-GELU, M=1024 K=768 N=3072 (tuned kerne
                   16384x4096x1024, next to the two plain GEMMs
        copy       plain device copy of 256 MiB (counter calibration: reads and
                   writes exactly 268435456 bytes each)
+       operands   gemm5 and gemm5g on random operands and on operands that are
+                  all zero (same instructions and traffic, no switching in the
+                  data paths): what the chip's power management costs the kernel
+       mfma_ceiling  v_mfma_f32_32x32x16_f16 back to back on register operands,
+                  no memory access in the loop, 8 wavefronts per CU: the rate the
+                  matrix cores sustain on zero and on random operands, alone and
+                  with 4 / 8 independent fp32 FMAs behind every MFMA
 Each call goes through the C-ABI via the C++ driver's timing helpers.
 """
 import ctypes
@@ -94,6 +101,21 @@ def main():
                                         1.0, 0.0, 0)
         torch.cuda.synchronize()
         print("ln pair 16384x1024x1024 -> 16384x4096x1024 x", iters)
+    elif what == "operands":
+        for (m, n, k, act, bias, label) in ((16384, 1024, 4096, 0, 0, "gemm5"), (16384, 4096, 1024, 1, 1, "gemm5g")):
+            pick(m, n, k, act)
+            for rep in range(2):
+                rnd = drv.homTimeGemm(m, n, k, act, bias, idx.value + 1, sk.value, iters, 3) * 1e3
+                zero = drv.homTimeGemmZeroOperands(m, n, k, act, bias, idx.value + 1, sk.value, iters, 3) * 1e3
+                tf = lambda us: 2.0 * m * n * k / us / 1e6
+                print(f"{label} {lib.homGemmManifestName(idx.value).decode()}: random operands {rnd:.2f} us "
+                      f"({tf(rnd):.0f} TFLOP/s), zero operands {zero:.2f} us ({tf(zero):.0f} TFLOP/s)", flush=True)
+    elif what == "mfma_ceiling":
+        for valu in (0, 4, 8):
+            for rnd in (0, 1, 0, 1):
+                tf = drv.homMfmaCeilingProbe(rnd, valu)
+                print(f"mfma only loop, {valu} fp32 FMAs per MFMA, {'random' if rnd else 'zero'} operands: "
+                      f"{tf:.0f} TFLOP/s = {tf / 2500:.3f} of the 2.5 PFLOP/s peak", flush=True)
     elif what == "copy":
         import torch
         src = torch.ones(128 * 1024 * 1024, dtype=torch.float16, device="cuda")
