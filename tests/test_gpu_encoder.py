@@ -289,6 +289,38 @@ def test_captured_split_k_graph_survives_scratch_growth(gpu, rt, synth):
         enc.close()
 
 
+def test_encoders_in_flight_on_separate_streams(gpu, rt, synth):
+    """Independent encoder instances (own buffers, stream and captured graph) replayed round-robin without
+    synchronising in between: every instance must keep producing its eager result.  None of their calls may use
+    the library's shared scratch (no split-K, no folded layer norm); that is checked, not assumed."""
+    bert = importlib.import_module("hands-on-mlir_amd.bert")
+    drv = rt.load_driver()
+    models = [synth.bert_encoder(layers=2, hidden=128, heads=2, ffn=512, bs=3, seq=64, vocab=1000, config=40 + i)
+              for i in range(3)]
+    encs, want = [], []
+    try:
+        for m in models:
+            e = bert.BertEncoder(2, 128, 2, 512, 3, 64, 1000, gemm_mode=1, gelu_form="erf")
+            encs.append(e)
+            e.load(m)
+            e.set_inputs(ids=m["ids"], mask=m["mask"])
+            assert all(split == 1 for _, split in e.gemm_choices().values())
+            e.forward()
+            want.append(e.output())
+            e.capture()
+        assert not np.array_equal(want[0], want[1])
+        for _ in range(20):
+            for e in encs:
+                e.replay()
+        for e in encs:
+            assert drv.homBertSync(e.h) == 0
+        for e, w in zip(encs, want):
+            assert np.array_equal(e.output(), w)
+    finally:
+        for e in encs:
+            e.close()
+
+
 def test_bert_base_b8_s128(gpu, oracle, synth):
     bert = importlib.import_module("hands-on-mlir_amd.bert")
     model = synth.bert_encoder()
