@@ -7,6 +7,7 @@ for the whole tensor whatever its size: column-sum checksums for GEMM, constant-
 and key-permutation invariance for attention, idempotence and unit statistics for
 layer norm, commutativity for add.  Tolerances are the ones of test_gpu_parity.
 """
+import ctypes
 import importlib
 
 import numpy as np
@@ -165,3 +166,19 @@ def test_elementwise_gather_cu_seqlens_bert_large_shapes(gpu, rt, oracle):
     cu = torch.empty(33, dtype=torch.int32, device="cuda")
     gpu.thrustCuSeqLenI64(*M(tm).args(), *M(cu).args())
     assert np.array_equal(host(cu), np.concatenate([[0], np.cumsum(lens)]).astype(np.int32))
+
+
+def test_driver_measurement_helpers(gpu, rt):
+    """The probes behind the figures on operand-dependent matrix-core rates run and give plausible numbers
+    (their exact values are a property of the box; the relations asserted here are kept loose)."""
+    drv = rt.load_driver()
+    zero, rnd = drv.homMfmaCeilingProbe(0, 0), drv.homMfmaCeilingProbe(1, 0)
+    assert 300 < rnd < 2600 and 300 < zero < 2600, (zero, rnd)
+    assert zero >= 0.9 * rnd, (zero, rnd)
+    assert 300 < drv.homMfmaCeilingProbe(1, 4) < 2600
+    idx, sk = ctypes.c_int64(), ctypes.c_int32()
+    gpu.homGemmSelect(ROWS, 1024, 4096, 0, ctypes.byref(idx), ctypes.byref(sk))
+    t_rnd = drv.homTimeGemm(ROWS, 1024, 4096, 0, 0, idx.value + 1, sk.value, 10, 3)
+    t_zero = drv.homTimeGemmZeroOperands(ROWS, 1024, 4096, 0, 0, idx.value + 1, sk.value, 10, 3)
+    assert 0.03 < t_zero < 1.0 and 0.03 < t_rnd < 1.0, (t_zero, t_rnd)
+    assert t_zero <= 1.1 * t_rnd, (t_zero, t_rnd)
