@@ -323,6 +323,11 @@ def main():
     kernels["bert_base_masked_lm_b8_s128"] = {"ms": mlm_ms, "sequences/s": d["bs"] / (mlm_ms * 1e-3),
                                               "TFLOP/s": (flops_forward + head_flops) / (mlm_ms * 1e-3) / 1e12}
 
+    # what a loop of nothing but MFMAs on register operands sustains on this box (zero / random operands): the
+    # ceiling any fp16 GEMM on random data sits under before a byte is moved
+    ceiling = {"zero_operands": drv.homMfmaCeilingProbe(0, 0) / PEAK_FP16_TFLOPS,
+               "random_operands": drv.homMfmaCeilingProbe(1, 0) / PEAK_FP16_TFLOPS}
+
     out = {
         "metric": METRIC, "value": seqs_per_s, "unit": "sequences/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms,
@@ -349,7 +354,8 @@ def main():
                      # the same launches as the nodes of a HIP graph (how the encoder runs them): the
                      # dependent-launch gap is 1.6 us there against 2.4 us on a stream
                      "us_per_launch_in_graph": g_graph_ms * 1e3,
-                     "frac_in_graph": g_flops / (g_graph_ms * 1e-3) / 1e12 / PEAK_FP16_TFLOPS},
+                     "frac_in_graph": g_flops / (g_graph_ms * 1e-3) / 1e12 / PEAK_FP16_TFLOPS,
+                     "frac_of_peak_of_an_mfma_only_loop": ceiling},
         "kernels": kernels,
     }
     if not args.no_cpu_baseline:
