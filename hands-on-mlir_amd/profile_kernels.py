@@ -8,6 +8,8 @@ tile (GEMM workloads only): run the manifest kernel whose name holds `_<tile>_`
 what:  gemm1      FFN1 GEMM + bias + tanh-GELU, M=1024 K=768 N=3072 (tuned kernel)
        gemm5      BERT-large FFN2 GEMM, M=16384 K=4096 N=1024
        gemm5g     BERT-large FFN1 GEMM + bias + erf-GELU, M=16384 K=1024 N=4096
+       gemm_skinny  the skinny split-K stress case, M=64 K=4096 N=1024 (two
+                  kernels per call: the K slices, then their reduction)
        layernorm  in-place layer norm, 16384 x 1024, the same tensor launch after
                   launch (it stays in the 256 MB Infinity Cache: a cache rate)
        layernorm_cold  the same over 24 tensors walked round-robin (805 MB:
@@ -67,6 +69,10 @@ def main():
         pick(16384, 4096, 1024, 1)
         ms = drv.homTimeGemm(16384, 4096, 1024, 1, 1, idx.value + 1, sk.value, iters, 3)
         print(f"gemm5g {lib.homGemmManifestName(idx.value).decode()} splitK {sk.value}: {ms * 1e3:.2f} us")
+    elif what == "gemm_skinny":
+        pick(64, 1024, 4096, 0)
+        ms = drv.homTimeGemm(64, 1024, 4096, 0, 0, idx.value + 1, sk.value, iters, 3)
+        print(f"gemm_skinny {lib.homGemmManifestName(idx.value).decode()} splitK {sk.value}: {ms * 1e3:.2f} us")
     elif what == "layernorm":
         print(f"layernorm 16384x1024: {drv.homTimeLayernorm(16384, 1024, 0, iters, 3) * 1e3:.2f} us")
     elif what == "layernorm_cold":
