@@ -79,6 +79,11 @@ class BertEncoder:
     def capture(self, from_ids=True):
         assert self.drv.homBertCapture(self.h, int(from_ids)) == 0
 
+    @property
+    def stream(self):
+        """The hipStream_t (as an integer) this encoder's calls are enqueued on."""
+        return self.drv.homBertGetStream(self.h)
+
     def replay(self):
         assert self.drv.homBertReplay(self.h) == 0
 

@@ -420,6 +420,7 @@ DRV_EXPORT void homBertDestroy(HomBertEncoder *e) {
     (void)hipGraphDestroy(e->graph);
   if (e->stream) {
     (void)hipStreamSynchronize(e->stream);
+    homReleaseStreamScratch(e->stream);
     (void)hipStreamDestroy(e->stream);
   }
   if (e->evStart)
@@ -545,6 +546,11 @@ DRV_EXPORT int homBertReplay(HomBertEncoder *e) {
                                                                           : -1;
 }
 
+// The stream the encoder's calls are enqueued on (a hipStream_t).
+DRV_EXPORT void *homBertGetStream(HomBertEncoder *e) {
+  return static_cast<void *>(e->stream);
+}
+
 DRV_EXPORT int homBertSync(HomBertEncoder *e) {
   return hipOk(hipStreamSynchronize(e->stream), "hipStreamSynchronize") ? 0 : -1;
 }
@@ -653,6 +659,7 @@ struct Timer {
       (void)hipEventDestroy(b);
     if (s) {
       (void)hipStreamSynchronize(s);
+      homReleaseStreamScratch(s);
       (void)hipStreamDestroy(s);
     }
   }

@@ -16,7 +16,14 @@ struct ScratchBuf {
   void *ptr = nullptr;
   size_t bytes = 0;
 };
-ScratchBuf g_scratch[kNumSlots];
+// One set of slots per stream that has asked for scratch: what is in flight on
+// two streams at once must not share partial results.
+struct StreamScratch {
+  hipStream_t stream = nullptr;
+  bool inUse = true;
+  ScratchBuf slot[kNumSlots];
+};
+std::vector<StreamScratch> g_scratch;
 std::vector<void *> g_retired; // replaced scratch buffers, kept allocated
 int g_scratchGeneration = 0;
 } // namespace
@@ -72,8 +79,32 @@ const DeviceInfo &deviceInfo() {
 
 int libraryScratchGeneration() { return g_scratchGeneration; }
 
+void releaseStreamScratch(hipStream_t s) {
+  for (StreamScratch &e : g_scratch)
+    if (e.inUse && e.stream == s && s != nullptr)
+      e.inUse = false;
+}
+
 void *libraryScratch(ScratchSlot slot, size_t bytes, bool zero) {
-  ScratchBuf &b = g_scratch[slot];
+  StreamScratch *mine = nullptr, *spare = nullptr;
+  for (StreamScratch &s : g_scratch) {
+    if (s.inUse && s.stream == g_stream)
+      mine = &s;
+    else if (!s.inUse && !spare)
+      spare = &s;
+  }
+  if (!mine) {
+    // a set that a finished stream gave back (releaseStreamScratch) serves the
+    // next new stream, buffers included
+    if (!spare) {
+      g_scratch.emplace_back();
+      spare = &g_scratch.back();
+    }
+    mine = spare;
+    mine->stream = g_stream;
+    mine->inUse = true;
+  }
+  ScratchBuf &b = mine->slot[slot];
   if (bytes <= b.bytes)
     return b.ptr;
   // Growing never frees the old buffer: queued kernels and captured graphs

@@ -94,8 +94,10 @@ struct DeviceInfo {
 };
 const DeviceInfo &deviceInfo();
 
-// Grow-only device scratch, one buffer per slot.  Slot kWorkspace holds
-// split-K partial tiles, kTemp the temporaries of the layer-norm GEMM pair.
+// Grow-only device scratch, one buffer per slot and per stream the library has
+// been pointed at (setStream): calls in flight on different streams do not
+// share partial results.  Slot kWorkspace holds split-K partial tiles, kTemp
+// the temporaries of the layer-norm GEMM pair.
 // A buffer that has been handed out is never freed while the process lives:
 // kernels already enqueued, and HIP graphs captured earlier, keep its address
 // in their arguments.  When a slot must grow, a new buffer of at least twice
@@ -107,5 +109,10 @@ enum ScratchSlot { kWorkspace = 0, kCounters = 1, kTemp = 2, kNumSlots = 3 };
 void *libraryScratch(ScratchSlot slot, size_t bytes, bool zero);
 // Number of times any slot has been replaced by a larger buffer (tests).
 int libraryScratchGeneration();
+// The caller is done with stream `s` (everything enqueued on it has finished
+// and no graph captured on it will be replayed): its buffers go to the next
+// stream that asks.  Without this call they stay with `s` until the process
+// ends.  The null stream's set is never given away.
+void releaseStreamScratch(hipStream_t s);
 
 } // namespace hom

@@ -187,6 +187,9 @@ void homSetStream(void *hipStream) {
   setStream(static_cast<hipStream_t>(hipStream));
 }
 void *homGetStream(void) { return static_cast<void *>(stream()); }
+void homReleaseStreamScratch(void *hipStream) {
+  releaseStreamScratch(static_cast<hipStream_t>(hipStream));
+}
 void homSetErrorMode(int32_t mode) { setErrorMode(mode == 1 ? 1 : 0); }
 const char *homGetLastError(void) { return takeLastError(); }
 int32_t homScratchGeneration(void) { return libraryScratchGeneration(); }

@@ -267,16 +267,24 @@ def test_captured_split_k_graph_survives_scratch_growth(gpu, rt, synth):
         enc.capture()
         enc.replay()
         assert np.array_equal(enc.output(), eager)
-        # a split-K GEMM whose partial tiles (2048 x 2048 x 4 slices x 4 B = 64 MiB) exceed anything
-        # the encoder asked for: the workspace slot is replaced by a larger buffer
+        # split-K GEMMs on the encoder's stream (the library keeps one workspace per stream) whose partial
+        # tiles exceed what the stream has asked for so far: the slot is replaced by a larger buffer
         before = gpu.homScratchGeneration()
         M = rt.MemRef.from_tensor
-        ta = torch.randn((1, 2048, 512), device="cuda").half()
-        tb = (torch.randn((1, 512, 2048), device="cuda") * 0.05).half()
-        td = torch.zeros((1, 2048, 2048), dtype=torch.float16, device="cuda")
-        gpu.cutlassGemmF16(*M(ta).args(), False, *M(tb).args(), False, *M(td).args(), *M(td).args(),
-                           0, 1.0, 0.0, number[tile], 4)
-        torch.cuda.synchronize()
+        prev = gpu.homGetStream()
+        gpu.homSetStream(enc.stream)
+        try:
+            for side in (2048, 4096):   # 64 MiB, then 256 MiB of partial tiles (4 slices of fp32)
+                ta = torch.randn((1, side, 512), device="cuda").half()
+                tb = (torch.randn((1, 512, side), device="cuda") * 0.05).half()
+                td = torch.zeros((1, side, side), dtype=torch.float16, device="cuda")
+                gpu.cutlassGemmF16(*M(ta).args(), False, *M(tb).args(), False, *M(td).args(), *M(td).args(),
+                                   0, 1.0, 0.0, number[tile], 4)
+                torch.cuda.synchronize()
+                if gpu.homScratchGeneration() > before:
+                    break
+        finally:
+            gpu.homSetStream(prev)
         assert gpu.homScratchGeneration() > before, "the workspace did not grow: the test tests nothing"
         # fill freshly allocated memory so that a dangling workspace would not go unnoticed
         junk = [torch.full((8 << 20,), float("nan"), dtype=torch.float32, device="cuda") for _ in range(4)]
@@ -291,10 +299,13 @@ def test_captured_split_k_graph_survives_scratch_growth(gpu, rt, synth):
 
 def test_encoders_in_flight_on_separate_streams(gpu, rt, synth):
     """Independent encoder instances (own buffers, stream and captured graph) replayed round-robin without
-    synchronising in between: every instance must keep producing its eager result.  None of their calls may use
-    the library's shared scratch (no split-K, no folded layer norm); that is checked, not assumed."""
+    synchronising in between: every instance must keep producing its eager result.  Two GEMM roles are pinned to
+    split-K kernels, whose partial tiles live in scratch the library allocates: it keeps one set per stream, so the
+    instances in flight do not overwrite each other's partial results."""
     bert = importlib.import_module("hands-on-mlir_amd.bert")
     drv = rt.load_driver()
+    number = {n: i + 1 for i, n, _, _ in rt.manifest()}
+    tile = "hom_gfx950_mfma_f16_s32x32x16gemm_f16_64x64_64x2r2_w2x2_nn_align8_linear"
     models = [synth.bert_encoder(layers=2, hidden=128, heads=2, ffn=512, bs=3, seq=64, vocab=1000, config=40 + i)
               for i in range(3)]
     encs, want = [], []
@@ -304,10 +315,12 @@ def test_encoders_in_flight_on_separate_streams(gpu, rt, synth):
             encs.append(e)
             e.load(m)
             e.set_inputs(ids=m["ids"], mask=m["mask"])
-            assert all(split == 1 for _, split in e.gemm_choices().values())
+            e.set_gemm_choice("out", number[tile], 2)
+            e.set_gemm_choice("ffn2", number[tile], 4)
             e.forward()
             want.append(e.output())
             e.capture()
+        assert len({e.stream for e in encs}) == len(encs)
         assert not np.array_equal(want[0], want[1])
         for _ in range(20):
             for e in encs:
