@@ -695,3 +695,88 @@ def test_alloc_family_and_constant_loader(gpu, rt, tmp_path, monkeypatch):
             src = (vals * scale).astype(np.float16 if idx == 5 else np.float32)
             assert np.array_equal(host(out), src.astype(np.float16 if dt == torch.float16 else np.float32))
             gpu.deallocNVGPUF16(m.rank, m.descriptor)
+
+
+# ------------------------------------------------------ randomised sweeps --
+def test_gemm_randomised_sweep(gpu, rt, oracle):
+    """Seeded random problems over every manifest kernel: ragged M / N / K, whole numbers of slabs, split-K, and the
+    four source forms (none, bias row, residual in place, separate full matrix) with alpha / beta other than 1.
+    Problems an aligned kernel cannot take are refused by the library's argument check (the reference's
+    can_implement) and skipped."""
+    g = np.random.default_rng(2024)
+    man = rt.manifest()
+    M_ = rt.MemRef.from_tensor
+    compared = 0
+    gpu.homSetErrorMode(1)
+    try:
+        for _ in range(500):
+            idx, name, act, align = man[g.integers(len(man))]
+            epi = "gelu_tanh" if "gelutanh" in name else ("gelu_erf" if act else "linear")
+            M, N, K = (int(g.integers(1, 520)) for _ in range(3))
+            if align == 8 and g.random() < 0.8:
+                N, K = max(8, N // 8 * 8), max(8, K // 8 * 8)
+            if g.random() < 0.15:
+                K = int(g.integers(1, 24)) * 64
+            sk = int(g.choice([1, 1, 2, 3, 5]))
+            mode = int(g.integers(4))
+            alpha = float(g.choice([1.0, 1.0, 0.5, 2.0]))
+            beta = 0.0 if mode == 0 else float(g.choice([1.0, 1.0, 0.5]))
+            A = g.standard_normal((1, M, K)).astype(np.float16)
+            B = (g.standard_normal((1, K, N)) * 0.1).astype(np.float16)
+            C = None if mode == 0 else g.standard_normal((1, 1 if mode == 1 else M, N)).astype(np.float16)
+            ta, tb = dev(A), dev(B)
+            td = dev(C) if mode == 2 else torch.zeros((1, M, N), dtype=torch.float16, device="cuda")
+            tc = td if mode in (0, 2) else dev(C)
+            gpu.homGetLastError()
+            gpu.cutlassGemmF16(*M_(ta).args(), False, *M_(tb).args(), False, *M_(tc).args(), *M_(td).args(),
+                               act, alpha, beta, idx + 1, sk)
+            err = gpu.homGetLastError().decode()
+            if err:
+                assert "multiples of" in err, err
+                continue
+            want = oracle.gemm(A[0], B[0], None if C is None else np.broadcast_to(C[0], (M, N)).astype(np.float16),
+                               alpha=alpha, beta=beta, act=epi)
+            assert_close(host(td)[0], want, **GEMM_TOL,
+                         what=f"{name} {M}x{N}x{K} splitK={sk} source form {mode} alpha={alpha} beta={beta}")
+            compared += 1
+    finally:
+        gpu.homSetErrorMode(0)
+    assert compared >= 300
+
+
+def test_attention_and_layernorm_randomised_sweep(gpu, rt, oracle):
+    """Seeded random attention problems (every head size, ragged and empty sequences, larger score amplitudes) and
+    layer norms (in place, and with residual and affine parameters; row lengths off the vector width)."""
+    g = np.random.default_rng(2025)
+    M_ = rt.MemRef.from_tensor
+    for _ in range(150):
+        d = int(g.choice([64, 64, 64, 128, 192, 256]))
+        heads, bs, seq = int(g.integers(1, 5)), int(g.integers(1, 6)), int(g.integers(1, 300))
+        amp = float(g.choice([1.0, 1.0, 3.0]))
+        qkv = (g.standard_normal((bs, seq, 3 * heads * d)) * amp).astype(np.float16)
+        lens = g.integers(0, seq + 1, size=bs).astype(np.int32)
+        got, cu = run_attention(gpu, rt, qkv, lens, heads, float(1.0 / np.sqrt(d)))
+        want = oracle.attention(qkv, cu, heads, float(1.0 / np.sqrt(d)))
+        for b in range(bs):
+            assert_close(got[b, :lens[b]], want[b, :lens[b]], **GEMM_TOL,
+                         what=f"attention d={d} heads={heads} bs={bs} seq={seq} lens={lens.tolist()} amplitude {amp}")
+            assert not got[b, lens[b]:].any()
+    for _ in range(150):
+        rows = int(g.integers(1, 300))
+        hidden = int(g.choice([8, 64, 96, 128, 760, 768, 1000, 1024, 2048, 3000, 4096, 5000]))
+        x = (g.standard_normal((rows, hidden)) * float(g.choice([1.0, 10.0])) + float(g.choice([0.0, 3.0])))
+        x = x.astype(np.float16)
+        eps = float(g.choice([1e-12, 1e-5]))
+        if g.integers(2):
+            res = g.standard_normal((rows, hidden)).astype(np.float16)
+            gamma = (1 + 0.02 * g.standard_normal(hidden)).astype(np.float16)
+            beta = (0.02 * g.standard_normal(hidden)).astype(np.float16)
+            tx, tr, tg, tb = dev(x), dev(res), dev(gamma), dev(beta)
+            to = torch.zeros_like(tx)
+            gpu.homAddLayernormF16(*M_(tx).args(), *M_(tr).args(), *M_(tg).args(), *M_(tb).args(), *M_(to).args(), eps)
+            got, want = host(to), oracle.layernorm_f16(x, eps, res, gamma, beta)
+        else:
+            tx = dev(x)
+            gpu.nvteLayernormF16(*M_(tx).args(), eps)
+            got, want = host(tx), oracle.layernorm_f16(x, eps)
+        assert_close(got, want, **LN_TOL, what=f"layer norm rows={rows} hidden={hidden} eps={eps}")
