@@ -780,3 +780,37 @@ def test_attention_and_layernorm_randomised_sweep(gpu, rt, oracle):
             gpu.nvteLayernormF16(*M_(tx).args(), eps)
             got, want = host(tx), oracle.layernorm_f16(x, eps)
         assert_close(got, want, **LN_TOL, what=f"layer norm rows={rows} hidden={hidden} eps={eps}")
+
+
+def test_library_selected_gemm_randomised_sweep(gpu, rt, oracle):
+    """Seeded random problems through the two entry points that let the library pick the kernel: cutlassGemmF16
+    with gemmNum == 0 (activation 0 / 1 / 2) and nvteGemmF16 (B as [N, K]; beta 0 or 1 in place; activation 1 is
+    the tanh form there).  Any M, N, K: the selection has to fall back to kernels that fit the alignment."""
+    g = np.random.default_rng(2026)
+    M_ = rt.MemRef.from_tensor
+    for it in range(300):
+        M, N, K = (int(g.integers(1, 600)) for _ in range(3))
+        if g.random() < 0.6:
+            N, K = max(8, N // 8 * 8), max(8, K // 8 * 8)
+        A = g.standard_normal((1, M, K)).astype(np.float16)
+        X = g.standard_normal((1, M, N)).astype(np.float16)
+        ta, td = dev(A), dev(X)
+        if it % 2 == 0:
+            act = int(g.integers(3))
+            B = (g.standard_normal((1, K, N)) * 0.1).astype(np.float16)
+            bias = g.standard_normal((1, 1, N)).astype(np.float16)
+            tb, tc = dev(B), dev(bias)
+            gpu.cutlassGemmF16(*M_(ta).args(), False, *M_(tb).args(), False, *M_(tc).args(), *M_(td).args(),
+                               act, 1.0, 1.0, 0, 1)
+            want = oracle.gemm(A[0], B[0], np.broadcast_to(bias[0], (M, N)).astype(np.float16), beta=1.0,
+                               act=("linear", "gelu_erf", "gelu_tanh")[act])
+            what = f"cutlassGemmF16 gemmNum=0 act={act} {M}x{N}x{K}"
+        else:
+            act, beta = int(g.integers(2)), float(g.integers(2))
+            Bt = (g.standard_normal((1, N, K)) * 0.1).astype(np.float16)
+            tb = dev(Bt)
+            gpu.nvteGemmF16(*M_(ta).args(), False, *M_(tb).args(), True, *M_(td).args(), *M_(td).args(),
+                            act, 1.0, beta, 0, 0)
+            want = oracle.gemm(A[0], Bt[0], X[0], beta=beta, act=("linear", "gelu_tanh")[act], b_is_nk=True)
+            what = f"nvteGemmF16 act={act} beta={beta} {M}x{N}x{K}"
+        assert_close(host(td)[0], want, **GEMM_TOL, what=what)
