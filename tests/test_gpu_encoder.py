@@ -297,6 +297,39 @@ def test_captured_split_k_graph_survives_scratch_growth(gpu, rt, synth):
         enc.close()
 
 
+def test_small_encoders_randomised_sweep(gpu, oracle, synth):
+    """Seeded random small encoders (1-3 layers, 1-4 heads, any FFN width that is a multiple of 8, any batch, sequence
+    length and vocabulary, ragged lengths) through every GEMM mode, both GELU forms and the folded-layer-norm call
+    list, eager and replayed, against the oracle."""
+    bert = importlib.import_module("hands-on-mlir_amd.bert")
+    g = np.random.default_rng(77)
+    for _ in range(60):
+        heads, layers, ffn = int(g.integers(1, 5)), int(g.integers(1, 4)), int(g.integers(1, 40)) * 8
+        hidden = heads * 64
+        bs, seq, vocab = int(g.integers(1, 6)), int(g.integers(1, 200)), int(g.integers(2, 2000))
+        mode, gelu = [(1, "erf"), (1, "tanh"), (0, "tanh")][int(g.integers(3))]
+        fold = bool(mode == 1 and gelu == "erf" and g.integers(2))
+        model = synth.bert_encoder(layers=layers, hidden=hidden, heads=heads, ffn=ffn, bs=bs, seq=seq, vocab=vocab,
+                                   config=int(g.integers(1000)))
+        model["lens"][:] = g.integers(1, seq + 1, size=bs)
+        model["mask"] = synth.mask_from_lengths(model["lens"], seq)
+        what = (f"layers={layers} hidden={hidden} ffn={ffn} bs={bs} seq={seq} vocab={vocab} mode={mode} gelu={gelu} "
+                f"fold={fold} lens={model['lens'].tolist()}")
+        enc = bert.BertEncoder(layers, hidden, heads, ffn, bs, seq, vocab, gemm_mode=mode, gelu_form=gelu,
+                               fold_layernorm=fold)
+        try:
+            enc.load(model)
+            enc.set_inputs(ids=model["ids"], mask=model["mask"])
+            enc.forward()
+            eager = enc.output()
+            check(eager, oracle_forward(oracle, model, gelu), model["lens"], what)
+            enc.capture()
+            enc.replay()
+            assert np.array_equal(enc.output(), eager), what
+        finally:
+            enc.close()
+
+
 def test_encoders_in_flight_on_separate_streams(gpu, rt, synth):
     """Independent encoder instances (own buffers, stream and captured graph) replayed round-robin without
     synchronising in between: every instance must keep producing its eager result.  Two GEMM roles are pinned to
