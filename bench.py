@@ -116,6 +116,10 @@ def main():
     import torch
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU")
+    # Under rocprofv3 the tracer itself has crashed (inside librocprofiler-sdk) on a few hundred replays of the
+    # folded-layer-norm graph while a few dozen were fine: keep that optional section short when a profiler's
+    # tool library is loaded, so that a traced default run completes.
+    traced = any("rocprofiler" in os.environ.get(k, "") for k in ("LD_PRELOAD", "ROCP_TOOL_LIBRARIES", "HSA_TOOLS_LIB"))
     rt = importlib.import_module("hands-on-mlir_amd.hom_runtime")
     synth = importlib.import_module("hands-on-mlir_amd.synth")
     bert = importlib.import_module("hands-on-mlir_amd.bert")
@@ -254,7 +258,7 @@ def main():
                                    gemm_mode=args.gemm_mode, gelu_form="erf", fold_layernorm=True)
             enc.load(big)
             enc.set_inputs(ids=big["ids"], mask=big["mask"])
-            fold_ms = enc.time(30, 15, graph=not args.eager)
+            fold_ms = enc.time(10 if traced else 30, 5 if traced else 15, graph=not args.eager)
             enc.close()
             kernels["bert_large_b32_s512_encoder_folded_layernorm"] = {
                 "ms": fold_ms, "sequences/s": 32 / (fold_ms * 1e-3), "TFLOP/s": big_flops / (fold_ms * 1e-3) / 1e12,
@@ -267,7 +271,8 @@ def main():
                                gemm_mode=args.gemm_mode, gelu_form="erf", fold_layernorm=True)
         enc.load(model)
         enc.set_inputs(ids=model["ids"], mask=model["mask"])
-        fold_ms = enc.time(args.steps, args.warmup, graph=not args.eager)
+        fold_ms = enc.time(min(args.steps, 20) if traced else args.steps, min(args.warmup, 5) if traced else args.warmup,
+                           graph=not args.eager)
         enc.close()
         kernels["bert_base_b8_s128_encoder_folded_layernorm"] = {
             "ms": fold_ms, "sequences/s": d["bs"] / (fold_ms * 1e-3),
