@@ -128,4 +128,82 @@ void *libraryScratch(ScratchSlot slot, size_t bytes, bool zero) {
   return p;
 }
 
+namespace {
+__global__ void xccOfWorkgroupKernel(unsigned int *out) {
+  unsigned int id;
+  asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(id));
+  if (threadIdx.x == 0)
+    out[blockIdx.x] = id & 15u;
+}
+
+enum class Placement { kUnknown, kRoundRobin, kOther };
+Placement g_placement = Placement::kUnknown;
+bool g_inKernelAllowed = false;
+int g_inKernelLaunches = 0;
+unsigned int *g_hostWords = nullptr; // [0] misplaced flag, [64..] the probe's output
+constexpr int kProbeGroups = 192;
+constexpr unsigned kXcds = 8;
+
+// Workgroup i of a launch runs on XCD (first + i) mod 8, whatever XCD the
+// launch starts on: checked on a few launches of grids that are not multiples
+// of eight (the start then differs from launch to launch).
+Placement measurePlacement(hipStream_t s) {
+  unsigned int *out = g_hostWords + 64;
+  for (int rep = 0; rep < 4; rep++) {
+    const int groups = kProbeGroups - rep;
+    xccOfWorkgroupKernel<<<dim3(groups), dim3(64), 0, s>>>(out);
+    if (hipGetLastError() != hipSuccess ||
+        hipStreamSynchronize(s) != hipSuccess)
+      return Placement::kOther;
+    for (int i = 0; i < groups; i++)
+      if (out[i] >= kXcds || out[i] != (out[0] + unsigned(i)) % kXcds)
+        return Placement::kOther;
+  }
+  return Placement::kRoundRobin;
+}
+} // namespace
+
+void setSplitKInKernel(bool on) { g_inKernelAllowed = on; }
+int splitKInKernelLaunches() { return g_inKernelLaunches; }
+
+bool splitKArrival(hipStream_t s, SplitKArrival *out) {
+  if (!g_inKernelAllowed || g_placement == Placement::kOther)
+    return false;
+  if (g_placement == Placement::kUnknown) {
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(s, &cap) != hipSuccess ||
+        cap != hipStreamCaptureStatusNone)
+      return false; // measuring needs a synchronisation
+    if (!g_hostWords) {
+      void *p = nullptr;
+      if (hipHostMalloc(&p, (64 + kProbeGroups) * sizeof(unsigned int),
+                        hipHostMallocMapped) != hipSuccess) {
+        (void)hipGetLastError();
+        g_placement = Placement::kOther;
+        return false;
+      }
+      g_hostWords = static_cast<unsigned int *>(p);
+      memset(g_hostWords, 0, (64 + kProbeGroups) * sizeof(unsigned int));
+    }
+    g_placement = measurePlacement(s);
+    if (g_placement != Placement::kRoundRobin)
+      return false;
+  }
+  if (*static_cast<volatile unsigned int *>(g_hostWords) != 0) {
+    g_placement = Placement::kOther;
+    HOM_CHECK_RET(false, false,
+                  "gemm: a split-K launch found the slices of one tile on "
+                  "different XCDs and its output may be wrong; later launches "
+                  "sum the slices with a second kernel");
+  }
+  void *w = libraryScratch(
+      kCounters, size_t(kMaxArrivalTiles) * sizeof(unsigned long long), true);
+  if (!w)
+    return false;
+  out->words = static_cast<unsigned long long *>(w);
+  out->misplaced = g_hostWords;
+  g_inKernelLaunches++;
+  return true;
+}
+
 } // namespace hom

@@ -115,4 +115,26 @@ int libraryScratchGeneration();
 // ends.  The null stream's set is never given away.
 void releaseStreamScratch(hipStream_t s);
 
+// In-kernel split-K reduction.  The K slices of a tile add one to the tile's
+// arrival word (slot kCounters, zero between launches: the slice that arrives
+// last sums the partial tiles and puts the word back to zero).  That slice
+// reads the others' partial tiles through its own L2, so the form is only
+// right when all slices of a tile run on one XCD; the launcher arranges that
+// from the round-robin placement of workgroups over the XCDs, which this
+// function measures once per process with a tiny kernel before it hands out
+// the words.  Returns nullptr -- sum with a second kernel instead -- while
+// `s` is being captured before that measurement has run, when the placement
+// is not the expected one, when a kernel has reported slices of one tile on
+// different XCDs (an error is recorded too), or unless setSplitKInKernel(true)
+// has switched the form on (it is off by default: measured, it is no faster
+// than the second kernel on the shapes the library splits by itself).
+constexpr int kMaxArrivalTiles = 8192;
+struct SplitKArrival {
+  unsigned long long *words; // [kMaxArrivalTiles]
+  unsigned int *misplaced;   // host-visible; kernels set it to 1 on a violation
+};
+bool splitKArrival(hipStream_t s, SplitKArrival *out);
+void setSplitKInKernel(bool on);
+int splitKInKernelLaunches(); // launches that used the in-kernel form (tests)
+
 } // namespace hom

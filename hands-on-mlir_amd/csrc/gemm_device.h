@@ -72,6 +72,11 @@ struct GemmParams {
   const _Float16 *C;
   _Float16 *D;
   float *workspace; // split-K partial tiles (null when gridDim.y == 1)
+  // In-kernel split-K reduction (null: a second kernel sums the slices): one
+  // arrival word per tile, and the host-visible word that reports slices of
+  // one tile found on different XCDs.
+  unsigned long long *tileArrivals;
+  unsigned int *misplaced;
   int M, N, K;
   int64_t lda, ldb, ldc, ldd;
   int cRowPeriod;
@@ -849,6 +854,113 @@ __device__ __forceinline__ void storePartial(const GemmParams &p,
       }
 }
 
+// In-kernel form of the split-K reduction, first half: this workgroup's
+// partial tile is in the workspace; count it in the tile's arrival word and
+// tell whether it was the last of the tile's slices to get there.  The last
+// one sums all the partial tiles (sumPartials) and finishes the tile; the
+// others are done with it.  No workgroup ever waits for another.
+//
+// All slices of a tile run on one XCD (the launcher's condition), so they
+// share an L2.  A slice's stores are in that L2 once its vmcnt has drained
+// (the vector L1 writes through); the barrier extends that to the workgroup,
+// and the atomic that follows goes to the same L2.  The last arriver drops its
+// L1 (buffer_inv sc0) so that its loads come from the L2 -- the lines could
+// only be in its L1 by accident of an earlier tile, but an accident is enough.
+// The arrival word also counts the slices per XCD (seven bits each above the
+// eight-bit total): a last arriver that does not find every slice on its own
+// XCD raises the host-visible flag, the library's check that the placement it
+// relies on held.  The word goes back to zero for the next launch.
+// `lds` is any four bytes of LDS nobody else uses between the two barriers.
+__device__ __forceinline__ bool arriveAtTile(const GemmParams &p, int tile,
+                                             int numSlices, int tid,
+                                             void *lds) {
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  volatile uint32_t *verdict = static_cast<volatile uint32_t *>(lds);
+  if (tid == 0) {
+    uint32_t xcc;
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
+    xcc &= 7u;
+    const unsigned long long mine = 1ull | (1ull << (8 + 7 * xcc));
+    const unsigned long long seen =
+        __hip_atomic_fetch_add(&p.tileArrivals[tile], mine, __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT) +
+        mine;
+    const bool last = uint32_t(seen & 255u) == uint32_t(numSlices);
+    if (last) {
+      if (uint32_t((seen >> (8 + 7 * xcc)) & 127u) != uint32_t(numSlices))
+        __hip_atomic_store(p.misplaced, 1u, __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_SYSTEM);
+      __hip_atomic_store(&p.tileArrivals[tile], 0ull, __ATOMIC_RELAXED,
+                         __HIP_MEMORY_SCOPE_AGENT);
+    }
+    *verdict = last ? 1u : 0u;
+  }
+  __syncthreads();
+  const bool last = __builtin_amdgcn_readfirstlane(int(*verdict)) != 0;
+  __syncthreads(); // the epilogue's strips may overwrite the verdict
+  if (last)
+    asm volatile("buffer_inv sc0\n\ts_waitcnt vmcnt(0)" ::: "memory");
+  return last;
+}
+
+// Second half: the tile's partial tiles, added in slice order starting from
+// zero -- the sum splitKReduceKernel forms, bit for bit.
+template <int MI, int NI, int THREADS>
+__device__ __forceinline__ void sumPartials(const GemmParams &p,
+                                            float16v (&acc)[MI][NI], int tile,
+                                            int numSlices, int tid) {
+  constexpr int ACC_V4 = MI * NI * 4;
+#pragma unroll
+  for (int i = 0; i < MI; i++)
+#pragma unroll
+    for (int j = 0; j < NI; j++)
+#pragma unroll
+      for (int e = 0; e < 16; e++)
+        acc[i][j][e] = 0.f;
+  const float4v *part = reinterpret_cast<const float4v *>(p.workspace) +
+                        int64_t(tile) * numSlices * (ACC_V4 * THREADS) + tid;
+  // Loads of up to AHEAD slices are in flight before the first add: one
+  // workgroup walks all the slices, and a small tile has only a few loads per
+  // slice to hide the L2's latency behind.
+  constexpr int AHEAD = ACC_V4 <= 4 ? 4 : ACC_V4 <= 8 ? 2 : 1;
+  int s = 0;
+  if constexpr (AHEAD > 1) {
+    for (; s + AHEAD <= numSlices; s += AHEAD, part += AHEAD * ACC_V4 * THREADS) {
+      float4v v[AHEAD][ACC_V4];
+#pragma unroll
+      for (int u = 0; u < AHEAD; u++)
+#pragma unroll
+        for (int q = 0; q < ACC_V4; q++)
+          v[u][q] = part[(u * ACC_V4 + q) * THREADS];
+#pragma unroll
+      for (int u = 0; u < AHEAD; u++) // slice order
+#pragma unroll
+        for (int i = 0; i < MI; i++)
+#pragma unroll
+          for (int j = 0; j < NI; j++)
+#pragma unroll
+            for (int g = 0; g < 4; g++)
+#pragma unroll
+              for (int e = 0; e < 4; e++)
+                acc[i][j][g * 4 + e] += v[u][(i * NI + j) * 4 + g][e];
+    }
+  }
+  for (; s < numSlices; s++, part += ACC_V4 * THREADS) {
+#pragma unroll
+    for (int i = 0; i < MI; i++)
+#pragma unroll
+      for (int j = 0; j < NI; j++)
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+          const float4v v = part[((i * NI + j) * 4 + g) * THREADS];
+#pragma unroll
+          for (int e = 0; e < 4; e++)
+            acc[i][j][g * 4 + e] += v[e];
+        }
+  }
+}
+
 template <int BM, int BN, int WM, int WN, int EPI, int VEC>
 __global__ __launch_bounds__(WM *WN *kWave) void splitKReduceKernel(
     GemmParams p, int numSlices) {
@@ -993,6 +1105,7 @@ struct LaunchPlan {
   GemmParams p;
   int splitK;
   int64_t nTiles;
+  bool callerWorkspace; // partial tiles go to a buffer the caller brought
 };
 
 template <int BM, int BN, int BK>
@@ -1045,6 +1158,9 @@ Status planLaunch(const GemmProblem &pr, LaunchPlan *plan) {
   // (the row range a wavefront addresses with 32-bit offsets is at most BM rows)
   p.epiMode = epilogueFastMode(p, BM);
   p.workspace = nullptr;
+  p.tileArrivals = nullptr;
+  p.misplaced = nullptr;
+  plan->callerWorkspace = pr.workspace != nullptr;
   if (splitK > 1) {
     const size_t wsBytes =
         size_t(plan->nTiles) * splitK * size_t(BM) * BN * sizeof(float);

@@ -731,9 +731,17 @@ __global__ __launch_bounds__(WM *WN *kWave) void gemmPipeKernel(
     epilogueFold<MI, NI, WTM, WTN, EPI, BM, THREADS>(p, acc, m0, n0, waveM,
                                                      waveN, lane, wave, tid,
                                                      foldStat, smem);
-  } else if (numSlices > 1)
+  } else if (numSlices > 1) {
     storePartial<MI, NI, THREADS>(p, acc, tile, slice, numSlices, tid);
-  else
+    if constexpr (EPI < kEpiRowStats) {
+      if (p.tileArrivals != nullptr &&
+          arriveAtTile(p, tile, numSlices, tid, smem)) {
+        sumPartials<MI, NI, THREADS>(p, acc, tile, numSlices, tid);
+        epilogueAuto<MI, NI, WTM, WTN, EPI>(p, acc, m0, n0, waveM, waveN, lane,
+                                            wave, smem);
+      }
+    }
+  } else
     epilogueAuto<MI, NI, WTM, WTN, EPI>(p, acc, m0, n0, waveM, waveN, lane,
                                         wave, smem);
   vpid += gridDim.x;
@@ -785,7 +793,21 @@ Status launchPipe(const GemmProblem &pr, hipStream_t s) {
     gridX = std::max<int64_t>(kNumXcd, resident / plan.splitK / kNumXcd * kNumXcd);
   if (gridX > plan.nTiles)
     gridX = plan.nTiles;
-  const GemmParams &q = plan.p;
+  GemmParams q = plan.p;
+  // The slices of a tile are workgroups x, x + gridX, x + 2 gridX ... of the
+  // launch: with gridX a multiple of the XCD count they share an XCD, and the
+  // last of them to finish can sum the partial tiles itself.
+  bool sumInKernel = false;
+  if (plan.splitK > 1 && plan.splitK <= 64 && EPI < kEpiRowStats &&
+      !plan.callerWorkspace && gridX % kNumXcd == 0 &&
+      plan.nTiles <= kMaxArrivalTiles) {
+    SplitKArrival arr;
+    if (splitKArrival(s, &arr)) {
+      q.tileArrivals = arr.words;
+      q.misplaced = arr.misplaced;
+      sumInKernel = true;
+    }
+  }
   // (leading dimensions fit 31 bits: checked above)
   kernel<<<dim3((unsigned)gridX, (unsigned)plan.splitK), dim3(WM * WN * kWave),
            SMEM, s>>>(q.A, q.B, q.M, q.N, q.K, int(q.lda), int(q.ldb), q.tilesN,
@@ -794,7 +816,7 @@ Status launchPipe(const GemmProblem &pr, hipStream_t s) {
                           uint32_t(q.fullGroups) << 8,
                       q.groupMagic, q.kTilesPerSlice, q);
   HOM_HIP_RET(hipGetLastError(), Status::kInternal);
-  if (plan.splitK > 1)
+  if (plan.splitK > 1 && !sumInKernel)
     return launchReduce<BM, BN, WM, WN, EPI, 8>(plan, s);
   return Status::kSuccess;
 }

@@ -190,6 +190,8 @@ void *homGetStream(void) { return static_cast<void *>(stream()); }
 void homReleaseStreamScratch(void *hipStream) {
   releaseStreamScratch(static_cast<hipStream_t>(hipStream));
 }
+void homSetSplitKInKernel(int32_t on) { setSplitKInKernel(on != 0); }
+int32_t homSplitKInKernelLaunches(void) { return splitKInKernelLaunches(); }
 void homSetErrorMode(int32_t mode) { setErrorMode(mode == 1 ? 1 : 0); }
 const char *homGetLastError(void) { return takeLastError(); }
 int32_t homScratchGeneration(void) { return libraryScratchGeneration(); }

@@ -10,6 +10,10 @@ what:  gemm1      FFN1 GEMM + bias + tanh-GELU, M=1024 K=768 N=3072 (tuned kerne
        gemm5g     BERT-large FFN1 GEMM + bias + erf-GELU, M=16384 K=1024 N=4096
        gemm_skinny  the skinny split-K stress case, M=64 K=4096 N=1024 (two
                   kernels per call: the K slices, then their reduction)
+       splitk_ab  the two forms of the split-K reduction side by side (a second
+                  kernel / the last slice to finish, inside the GEMM kernel), in
+                  a replayed HIP graph, over split factors 1..16 of the skinny
+                  case and of two BERT-base shapes
        layernorm  in-place layer norm, 16384 x 1024, the same tensor launch after
                   launch (it stays in the 256 MB Infinity Cache: a cache rate)
        layernorm_cold  the same over 24 tensors walked round-robin (805 MB:
@@ -73,6 +77,26 @@ def main():
         pick(64, 1024, 4096, 0)
         ms = drv.homTimeGemm(64, 1024, 4096, 0, 0, idx.value + 1, sk.value, iters, 3)
         print(f"gemm_skinny {lib.homGemmManifestName(idx.value).decode()} splitK {sk.value}: {ms * 1e3:.2f} us")
+    elif what == "splitk_ab":
+        num = {n: i + 1 for i, n, _, _ in rt.manifest()}
+        stem = "hom_gfx950_mfma_f16_s32x32x16gemm_f16_%s_nn_align8_linear"
+        try:
+            for (m, n, k) in ((64, 1024, 4096), (1024, 768, 3072), (1024, 768, 768)):
+                for tile in ("64x64_64q3_w2x2", "64x64_64x2r2_w2x2", "128x128_64q3_w2x4"):
+                    row = []
+                    for sk in (1, 2, 3, 4, 6, 8, 12, 16):
+                        if k // 64 < 2 * sk:
+                            continue
+                        us = []
+                        for on in (0, 1):
+                            lib.homSetSplitKInKernel(on)
+                            us.append(min(drv.homTimeGemmInGraph(m, n, k, 0, 0, num[stem % tile], sk, 1000, 100)
+                                          for _ in range(2)) * 1e3)
+                        row.append(f"splitK {sk}: {us[0]:.2f} / {us[1]:.2f}")
+                    print(f"splitk_ab {m}x{n}x{k} {tile} (us, second kernel / in kernel)  " + "  ".join(row),
+                          flush=True)
+        finally:
+            lib.homSetSplitKInKernel(0)
     elif what == "layernorm":
         print(f"layernorm 16384x1024: {drv.homTimeLayernorm(16384, 1024, 0, iters, 3) * 1e3:.2f} us")
     elif what == "layernorm_cold":

@@ -814,3 +814,44 @@ def test_library_selected_gemm_randomised_sweep(gpu, rt, oracle):
             want = oracle.gemm(A[0], Bt[0], X[0], beta=beta, act=("linear", "gelu_tanh")[act], b_is_nk=True)
             what = f"nvteGemmF16 act={act} beta={beta} {M}x{N}x{K}"
         assert_close(host(td)[0], want, **GEMM_TOL, what=what)
+
+
+def test_gemm_split_k_summed_in_kernel_matches_second_kernel(gpu, rt, oracle):
+    """The optional in-kernel split-K reduction (the last slice of a tile to finish adds the partial
+    tiles) against the default second kernel: same sums in the same order, so outputs agree to the last
+    bit of fp16 (the epilogue's rounding may differ), run to run identical, and within the GEMM
+    tolerance of the oracle.  Launches whose grid does not keep a tile's slices on one XCD must stay on
+    the second kernel."""
+    g = np.random.default_rng(36)
+    used0 = gpu.homSplitKInKernelLaunches()
+    try:
+        for (M, N, K) in ((64, 1024, 4096), (512, 512, 1024), (200, 328, 1000), (1024, 768, 768)):
+            A = g.standard_normal((1, M, K)).astype(np.float16)
+            B = (g.standard_normal((1, K, N)) * 0.1).astype(np.float16)
+            C = g.standard_normal((1, M, N)).astype(np.float16)
+            want = oracle.gemm(A[0], B[0])
+            for tile in ("64x64_64q3_w2x2", "64x64_64x2r2_w2x2", "128x128_64x2r2_w2x4"):
+                for epi, act, beta in (("linear", 0, 0.0), ("linear", 0, 1.0), ("gelu", 1, 1.0)):
+                    num = knum(rt, tile, epi)
+                    for sk in (2, 3, 8):
+                        zero = np.zeros((1, M, N), np.float16)
+                        gpu.homSetSplitKInKernel(0)
+                        two = run_gemm(gpu, rt, A, B, C, zero, num, sk, beta=beta, act=act)
+                        gpu.homSetSplitKInKernel(1)
+                        before = gpu.homSplitKInKernelLaunches()
+                        one = run_gemm(gpu, rt, A, B, C, zero, num, sk, beta=beta, act=act)
+                        again = run_gemm(gpu, rt, A, B, C, zero, num, sk, beta=beta, act=act)
+                        what = f"{M}x{N}x{K} {tile} {epi} beta={beta} splitK={sk}"
+                        bm, bn = (int(v) for v in tile.split("_")[0].split("x"))
+                        tiles_n = -(-N // bn) * -(-M // bm)
+                        took = gpu.homSplitKInKernelLaunches() - before
+                        assert took == (2 if tiles_n % 8 == 0 else 0), what
+                        assert np.array_equal(one, again), what
+                        a, b = one.astype(np.float32), two.astype(np.float32)
+                        ulp = np.maximum(np.abs(b), 2.0 ** -14) * 2.0 ** -10
+                        assert (np.abs(a - b) <= ulp).all(), what
+                        if not beta and not act:
+                            assert_close(one[0], want, **GEMM_TOL, what=what)
+    finally:
+        gpu.homSetSplitKInKernel(0)
+    assert gpu.homSplitKInKernelLaunches() > used0
