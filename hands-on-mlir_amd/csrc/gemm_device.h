@@ -20,7 +20,9 @@
 //    columns of one row of D and the epilogue can use 64-bit accesses;
 //  * split-K: gridDim.y slices of K each store their fp32 partial tile to a
 //    workspace; a second, small kernel sums the slices in slice order
-//    (deterministic, fp32) and runs the epilogue.  Nothing spins or fences;
+//    (deterministic, fp32) and runs the epilogue.  Nothing spins or fences.
+//    Optionally (pipe kernels, slices of a tile on one XCD) the slice that
+//    finishes last forms the same sum inside the kernel: arriveAtTile();
 //  * workgroup ids are remapped so that each of the 8 XCDs (which receive
 //    consecutive ids round-robin and have private L2s) works on a contiguous
 //    run of tiles.
