@@ -139,6 +139,7 @@ __global__ void xccOfWorkgroupKernel(unsigned int *out) {
 enum class Placement { kUnknown, kRoundRobin, kOther };
 Placement g_placement = Placement::kUnknown;
 bool g_inKernelAllowed = false;
+bool g_inKernelAnyGrid = false;
 int g_inKernelLaunches = 0;
 unsigned int *g_hostWords = nullptr; // [0] misplaced flag, [64..] the probe's output
 constexpr int kProbeGroups = 192;
@@ -163,7 +164,17 @@ Placement measurePlacement(hipStream_t s) {
 }
 } // namespace
 
-void setSplitKInKernel(bool on) { g_inKernelAllowed = on; }
+void setSplitKInKernel(int mode) {
+  g_inKernelAllowed = mode != 0;
+  g_inKernelAnyGrid = mode == 2;
+  // Switching (in either direction) forgets a reported violation: the
+  // placement is measured again before the form is next used.
+  if (g_placement == Placement::kOther)
+    g_placement = Placement::kUnknown;
+  if (g_hostWords)
+    *static_cast<volatile unsigned int *>(g_hostWords) = 0;
+}
+bool splitKInKernelAnyGrid() { return g_inKernelAnyGrid; }
 int splitKInKernelLaunches() { return g_inKernelLaunches; }
 
 bool splitKArrival(hipStream_t s, SplitKArrival *out) {

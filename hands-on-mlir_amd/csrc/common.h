@@ -125,7 +125,7 @@ void releaseStreamScratch(hipStream_t s);
 // the words.  Returns nullptr -- sum with a second kernel instead -- while
 // `s` is being captured before that measurement has run, when the placement
 // is not the expected one, when a kernel has reported slices of one tile on
-// different XCDs (an error is recorded too), or unless setSplitKInKernel(true)
+// different XCDs (an error is recorded too), or unless setSplitKInKernel(1)
 // has switched the form on (it is off by default: measured, it is no faster
 // than the second kernel on the shapes the library splits by itself).
 constexpr int kMaxArrivalTiles = 8192;
@@ -134,7 +134,11 @@ struct SplitKArrival {
   unsigned int *misplaced;   // host-visible; kernels set it to 1 on a violation
 };
 bool splitKArrival(hipStream_t s, SplitKArrival *out);
-void setSplitKInKernel(bool on);
+// mode 0: off; 1: on; 2: on, and the launcher skips its own condition on the
+// grid (slices of a tile then land on different XCDs and the kernels' check
+// must report it: what the tests of that check use).
+void setSplitKInKernel(int mode);
+bool splitKInKernelAnyGrid();
 int splitKInKernelLaunches(); // launches that used the in-kernel form (tests)
 
 } // namespace hom

@@ -799,7 +799,8 @@ Status launchPipe(const GemmProblem &pr, hipStream_t s) {
   // last of them to finish can sum the partial tiles itself.
   bool sumInKernel = false;
   if (plan.splitK > 1 && plan.splitK <= 64 && EPI < kEpiRowStats &&
-      !plan.callerWorkspace && gridX % kNumXcd == 0 &&
+      !plan.callerWorkspace &&
+      (gridX % kNumXcd == 0 || splitKInKernelAnyGrid()) &&
       plan.nTiles <= kMaxArrivalTiles) {
     SplitKArrival arr;
     if (splitKArrival(s, &arr)) {

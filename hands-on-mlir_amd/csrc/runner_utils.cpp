@@ -190,7 +190,9 @@ void *homGetStream(void) { return static_cast<void *>(stream()); }
 void homReleaseStreamScratch(void *hipStream) {
   releaseStreamScratch(static_cast<hipStream_t>(hipStream));
 }
-void homSetSplitKInKernel(int32_t on) { setSplitKInKernel(on != 0); }
+void homSetSplitKInKernel(int32_t mode) {
+  setSplitKInKernel(mode == 2 ? 2 : (mode != 0 ? 1 : 0));
+}
 int32_t homSplitKInKernelLaunches(void) { return splitKInKernelLaunches(); }
 void homSetErrorMode(int32_t mode) { setErrorMode(mode == 1 ? 1 : 0); }
 const char *homGetLastError(void) { return takeLastError(); }

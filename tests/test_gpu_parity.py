@@ -855,3 +855,42 @@ def test_gemm_split_k_summed_in_kernel_matches_second_kernel(gpu, rt, oracle):
     finally:
         gpu.homSetSplitKInKernel(0)
     assert gpu.homSplitKInKernelLaunches() > used0
+
+
+def test_gemm_split_k_in_kernel_reports_misplaced_slices(gpu, rt, oracle):
+    """The device-side check behind the in-kernel split-K reduction.  Mode 2 drops the launcher's condition
+    on the grid, so with 6 tiles the slices of a tile run on different XCDs: the last arriver of each tile
+    must notice (the arrival word counts slices per XCD), the next split-K launch must report it, sum with
+    the second kernel from then on, and still be right.  Nothing faults or waits: only the values of the
+    misplaced launch are undefined."""
+    g = np.random.default_rng(37)
+    M, N, K = 200, 328, 1024
+    A = g.standard_normal((1, M, K)).astype(np.float16)
+    B = (g.standard_normal((1, K, N)) * 0.1).astype(np.float16)
+    want = oracle.gemm(A[0], B[0])
+    num = knum(rt, "128x128_64x2r2_w2x4")   # 2 x 3 tiles
+    zero = np.zeros((1, M, N), np.float16)
+    gpu.homSetErrorMode(1)
+    try:
+        gpu.homSetSplitKInKernel(2)
+        before = gpu.homSplitKInKernelLaunches()
+        run_gemm(gpu, rt, A, B, None, zero, num, 3)          # misplaced on purpose; output not looked at
+        assert gpu.homSplitKInKernelLaunches() == before + 1
+        assert gpu.homGetLastError() == b""
+        out = run_gemm(gpu, rt, A, B, None, zero, num, 3)    # finds the report, falls back
+        assert b"different XCDs" in gpu.homGetLastError()
+        assert gpu.homSplitKInKernelLaunches() == before + 1
+        assert_close(out[0], want, **GEMM_TOL, what="launch that reported the misplaced slices")
+        out = run_gemm(gpu, rt, A, B, None, zero, num, 3)    # stays on the second kernel, silently
+        assert gpu.homGetLastError() == b"" and gpu.homSplitKInKernelLaunches() == before + 1
+        assert_close(out[0], want, **GEMM_TOL, what="launch after the report")
+        # switching the form on again measures the placement afresh and uses it where the grid allows
+        gpu.homSetSplitKInKernel(1)
+        A2 = g.standard_normal((1, 256, K)).astype(np.float16)
+        B2 = (g.standard_normal((1, K, 512)) * 0.1).astype(np.float16)
+        out = run_gemm(gpu, rt, A2, B2, None, np.zeros((1, 256, 512), np.float16), num, 3)   # 2 x 4 tiles
+        assert gpu.homGetLastError() == b"" and gpu.homSplitKInKernelLaunches() == before + 2
+        assert_close(out[0], oracle.gemm(A2[0], B2[0]), **GEMM_TOL, what="after re-arming")
+    finally:
+        gpu.homSetSplitKInKernel(0)
+        gpu.homSetErrorMode(0)
