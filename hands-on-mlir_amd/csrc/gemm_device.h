@@ -878,7 +878,7 @@ __device__ __forceinline__ bool arriveAtTile(const GemmParams &p, int tile,
                                              void *lds) {
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
-  volatile uint32_t *verdict = static_cast<volatile uint32_t *>(lds);
+  volatile uint32_t *wasLast = static_cast<volatile uint32_t *>(lds);
   if (tid == 0) {
     uint32_t xcc;
     asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
@@ -896,11 +896,11 @@ __device__ __forceinline__ bool arriveAtTile(const GemmParams &p, int tile,
       __hip_atomic_store(&p.tileArrivals[tile], 0ull, __ATOMIC_RELAXED,
                          __HIP_MEMORY_SCOPE_AGENT);
     }
-    *verdict = last ? 1u : 0u;
+    *wasLast = last ? 1u : 0u;
   }
   __syncthreads();
-  const bool last = __builtin_amdgcn_readfirstlane(int(*verdict)) != 0;
-  __syncthreads(); // the epilogue's strips may overwrite the verdict
+  const bool last = __builtin_amdgcn_readfirstlane(int(*wasLast)) != 0;
+  __syncthreads(); // the epilogue's strips may overwrite that word
   if (last)
     asm volatile("buffer_inv sc0\n\ts_waitcnt vmcnt(0)" ::: "memory");
   return last;
