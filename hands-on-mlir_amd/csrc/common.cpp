@@ -138,8 +138,7 @@ __global__ void xccOfWorkgroupKernel(unsigned int *out) {
 
 enum class Placement { kUnknown, kRoundRobin, kOther };
 Placement g_placement = Placement::kUnknown;
-bool g_inKernelAllowed = false;
-bool g_inKernelAnyGrid = false;
+int g_inKernelMode = 3; // see setSplitKInKernel()
 int g_inKernelLaunches = 0;
 unsigned int *g_hostWords = nullptr; // [0] misplaced flag, [64..] the probe's output
 constexpr int kProbeGroups = 192;
@@ -165,8 +164,7 @@ Placement measurePlacement(hipStream_t s) {
 } // namespace
 
 void setSplitKInKernel(int mode) {
-  g_inKernelAllowed = mode != 0;
-  g_inKernelAnyGrid = mode == 2;
+  g_inKernelMode = mode;
   // Switching (in either direction) forgets a reported violation: the
   // placement is measured again before the form is next used.
   if (g_placement == Placement::kOther)
@@ -174,11 +172,11 @@ void setSplitKInKernel(int mode) {
   if (g_hostWords)
     *static_cast<volatile unsigned int *>(g_hostWords) = 0;
 }
-bool splitKInKernelAnyGrid() { return g_inKernelAnyGrid; }
+int splitKInKernelMode() { return g_inKernelMode; }
 int splitKInKernelLaunches() { return g_inKernelLaunches; }
 
 bool splitKArrival(hipStream_t s, SplitKArrival *out) {
-  if (!g_inKernelAllowed || g_placement == Placement::kOther)
+  if (g_inKernelMode == 0 || g_placement == Placement::kOther)
     return false;
   if (g_placement == Placement::kUnknown) {
     hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;

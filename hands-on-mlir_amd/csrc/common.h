@@ -125,20 +125,28 @@ void releaseStreamScratch(hipStream_t s);
 // the words.  Returns nullptr -- sum with a second kernel instead -- while
 // `s` is being captured before that measurement has run, when the placement
 // is not the expected one, when a kernel has reported slices of one tile on
-// different XCDs (an error is recorded too), or unless setSplitKInKernel(1)
-// has switched the form on (it is off by default: measured, it is no faster
-// than the second kernel on the shapes the library splits by itself).
+// different XCDs (an error is recorded too), or after setSplitKInKernel(0).
 constexpr int kMaxArrivalTiles = 8192;
 struct SplitKArrival {
   unsigned long long *words; // [kMaxArrivalTiles]
   unsigned int *misplaced;   // host-visible; kernels set it to 1 on a violation
 };
 bool splitKArrival(hipStream_t s, SplitKArrival *out);
-// mode 0: off; 1: on; 2: on, and the launcher skips its own condition on the
-// grid (slices of a tile then land on different XCDs and the kernels' check
-// must report it: what the tests of that check use).
+// mode 0: never; 1: wherever the launch keeps a tile's slices on one XCD;
+// 2: like 1, and the launcher skips that condition (slices then land on
+// different XCDs and the kernels' check must report it: what the tests of that
+// check use); 3 (the default): like 1, but only where it measured faster than
+// the second kernel (splitKInKernelPays()).
 void setSplitKInKernel(int mode);
-bool splitKInKernelAnyGrid();
+int splitKInKernelMode();
+// Measured on MI355X over tiles, shapes and split factors: the last arriver
+// walks its tile's slices alone, so the form pays with small tiles (a partial
+// tile of at most 32 KB), few slices, and a launch that is resident at once
+// with room to spare; otherwise the second kernel, which spreads the sum over
+// the whole chip, is as fast or faster.
+inline bool splitKInKernelPays(int tileElems, int slices, long long tiles) {
+  return tileElems <= 128 * 64 && slices <= 6 && tiles * slices <= 512;
+}
 int splitKInKernelLaunches(); // launches that used the in-kernel form (tests)
 
 } // namespace hom

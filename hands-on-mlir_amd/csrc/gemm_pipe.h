@@ -800,7 +800,9 @@ Status launchPipe(const GemmProblem &pr, hipStream_t s) {
   bool sumInKernel = false;
   if (plan.splitK > 1 && plan.splitK <= 64 && EPI < kEpiRowStats &&
       !plan.callerWorkspace &&
-      (gridX % kNumXcd == 0 || splitKInKernelAnyGrid()) &&
+      (gridX % kNumXcd == 0 || splitKInKernelMode() == 2) &&
+      (splitKInKernelMode() != 3 ||
+       splitKInKernelPays(BM * BN, plan.splitK, plan.nTiles)) &&
       plan.nTiles <= kMaxArrivalTiles) {
     SplitKArrival arr;
     if (splitKArrival(s, &arr)) {

@@ -191,7 +191,7 @@ void homReleaseStreamScratch(void *hipStream) {
   releaseStreamScratch(static_cast<hipStream_t>(hipStream));
 }
 void homSetSplitKInKernel(int32_t mode) {
-  setSplitKInKernel(mode == 2 ? 2 : (mode != 0 ? 1 : 0));
+  setSplitKInKernel(mode >= 0 && mode <= 3 ? mode : 3);
 }
 int32_t homSplitKInKernelLaunches(void) { return splitKInKernelLaunches(); }
 void homSetErrorMode(int32_t mode) { setErrorMode(mode == 1 ? 1 : 0); }

@@ -96,7 +96,7 @@ def main():
                     print(f"splitk_ab {m}x{n}x{k} {tile} (us, second kernel / in kernel)  " + "  ".join(row),
                           flush=True)
         finally:
-            lib.homSetSplitKInKernel(0)
+            lib.homSetSplitKInKernel(3)  # the default
     elif what == "layernorm":
         print(f"layernorm 16384x1024: {drv.homTimeLayernorm(16384, 1024, 0, iters, 3) * 1e3:.2f} us")
     elif what == "layernorm_cold":

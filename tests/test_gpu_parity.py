@@ -852,8 +852,21 @@ def test_gemm_split_k_summed_in_kernel_matches_second_kernel(gpu, rt, oracle):
                         assert (np.abs(a - b) <= ulp).all(), what
                         if not beta and not act:
                             assert_close(one[0], want, **GEMM_TOL, what=what)
+        # the default mode takes the in-kernel form only where it measured faster: small tiles,
+        # at most 6 slices, at most 512 workgroups
+        gpu.homSetSplitKInKernel(3)
+        A = g.standard_normal((1, 64, 4096)).astype(np.float16)
+        B = (g.standard_normal((1, 4096, 1024)) * 0.1).astype(np.float16)
+        want = oracle.gemm(A[0], B[0])
+        zero = np.zeros((1, 64, 1024), np.float16)
+        for tile, sk, expect in (("64x64_64x2r2_w2x2", 4, 1), ("64x64_64x2r2_w2x2", 8, 0),
+                                 ("128x128_64x2r2_w2x4", 2, 0), ("64x64_64q3_w2x2", 6, 1)):
+            before = gpu.homSplitKInKernelLaunches()
+            out = run_gemm(gpu, rt, A, B, None, zero, knum(rt, tile), sk)
+            assert gpu.homSplitKInKernelLaunches() - before == expect, (tile, sk)
+            assert_close(out[0], want, **GEMM_TOL, what=f"default mode {tile} splitK={sk}")
     finally:
-        gpu.homSetSplitKInKernel(0)
+        gpu.homSetSplitKInKernel(3)   # the default
     assert gpu.homSplitKInKernelLaunches() > used0
 
 
@@ -892,5 +905,5 @@ def test_gemm_split_k_in_kernel_reports_misplaced_slices(gpu, rt, oracle):
         assert gpu.homGetLastError() == b"" and gpu.homSplitKInKernelLaunches() == before + 2
         assert_close(out[0], oracle.gemm(A2[0], B2[0]), **GEMM_TOL, what="after re-arming")
     finally:
-        gpu.homSetSplitKInKernel(0)
+        gpu.homSetSplitKInKernel(3)   # the default
         gpu.homSetErrorMode(0)
