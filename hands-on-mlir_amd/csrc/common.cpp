@@ -205,8 +205,22 @@ bool splitKArrival(hipStream_t s, SplitKArrival *out) {
                   "different XCDs and its output may be wrong; later launches "
                   "sum the slices with a second kernel");
   }
-  void *w = libraryScratch(
-      kCounters, size_t(kMaxArrivalTiles) * sizeof(unsigned long long), true);
+  // The words of this stream's set.  Allocating them clears them with a
+  // synchronous memset, which a stream under capture must not see: a first use
+  // inside a capture sums with the second kernel instead.
+  constexpr size_t kWordBytes =
+      size_t(kMaxArrivalTiles) * sizeof(unsigned long long);
+  void *w = nullptr;
+  for (const StreamScratch &e : g_scratch)
+    if (e.inUse && e.stream == g_stream && e.slot[kCounters].bytes >= kWordBytes)
+      w = e.slot[kCounters].ptr;
+  if (!w) {
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(s, &cap) != hipSuccess ||
+        cap != hipStreamCaptureStatusNone)
+      return false;
+    w = libraryScratch(kCounters, kWordBytes, true);
+  }
   if (!w)
     return false;
   out->words = static_cast<unsigned long long *>(w);
