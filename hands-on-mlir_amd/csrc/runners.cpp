@@ -241,11 +241,12 @@ bool selectGemm(int64_t M, int64_t N, int64_t K, int64_t activation,
       {128, 128, 2, 4, 2}, {128, 256, 2, 4, 2}, {256, 128, 4, 2, 2},
       {256, 256, 2, 4, 1},
   };
-  constexpr double kLaunchUs = 3.0, kReduceLaunchUs = 2.5;
+  constexpr double kLaunchUs = 3.0, kReduceLaunchUs = 2.5, kInKernelSumUs = 1.0;
   constexpr double kUsPerOutputSlab = 2.234e-5;
   constexpr double kL2BytesPerUs = 24.0e6;
   constexpr double kSlabFloorUs = 0.17;
   constexpr double kReduceBytesPerUs = 3.0e6; // partial tiles, written + read
+  constexpr double kInKernelBytesPerUs = 9.0e6; // the same, staying in one L2
   const double epiNsPerOutput = epi == Epilogue::kLinear ? 0.045 : 0.12;
   const char *epiName = epi == Epilogue::kLinear
                             ? "linear"
@@ -281,9 +282,16 @@ bool selectGemm(int64_t M, int64_t N, int64_t K, int64_t activation,
         double cost = kLaunchUs +
                       std::max(perSlice * kSlabFloorUs, compute + traffic) +
                       std::ceil(double(tiles) / cus) * area * epiNsPerOutput * 1e-3;
-        if (sp > 1)
-          cost += kReduceLaunchUs +
-                  double(tiles) * sp * area * 8.0 / kReduceBytesPerUs;
+        if (sp > 1) {
+          // (the in-kernel sum saves most of the second launch where the
+          // launcher will take it: same conditions as launchPipe)
+          const bool inKernel = splitKInKernelMode() != 0 && tiles % 8 == 0 &&
+                                (splitKInKernelMode() != 3 ||
+                                 splitKInKernelPays(t.tileM * t.tileN, sp, tiles));
+          cost += (inKernel ? kInKernelSumUs : kReduceLaunchUs) +
+                  double(tiles) * sp * area * 8.0 /
+                      (inKernel ? kInKernelBytesPerUs : kReduceBytesPerUs);
+        }
         if (cost < bestCost) {
           bestCost = cost;
           best = idxOf;
