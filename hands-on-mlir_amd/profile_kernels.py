@@ -8,8 +8,8 @@ tile (GEMM workloads only): run the manifest kernel whose name holds `_<tile>_`
 what:  gemm1      FFN1 GEMM + bias + tanh-GELU, M=1024 K=768 N=3072 (tuned kernel)
        gemm5      BERT-large FFN2 GEMM, M=16384 K=4096 N=1024
        gemm5g     BERT-large FFN1 GEMM + bias + erf-GELU, M=16384 K=1024 N=4096
-       gemm_skinny  the skinny split-K stress case, M=64 K=4096 N=1024 (two
-                  kernels per call: the K slices, then their reduction)
+       gemm_skinny  the skinny split-K stress case, M=64 K=4096 N=1024, as the
+                  library runs it (tuned kernel and split factor)
        splitk_ab  the two forms of the split-K reduction side by side (a second
                   kernel / the last slice to finish, inside the GEMM kernel), in
                   a replayed HIP graph, over split factors 1..16 of the skinny
