@@ -32,7 +32,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 
 def bert_shapes():
     shapes = []
-    for (hidden, ffn, rows) in [(768, 3072, (128, 1024, 2048, 4096)),      # base: b1..b32 x s128
+    for (hidden, ffn, rows) in [(768, 3072, (128, 256, 512, 1024, 2048, 4096)),  # base: b1, b2, b4 ... b32 x s128
                                 (1024, 4096, (128, 1024, 4096, 16384))]:  # large, up to b32 x s512
         for m in rows:
             for act_gelu in (1, 2):
