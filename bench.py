@@ -317,6 +317,15 @@ def main():
             "note": "throughput of independent batches on separate streams; the headline value is one forward "
                     "after the other, the reference's protocol"}
 
+    # What the chain of launches itself costs: 88 empty kernels as the nodes of one replayed graph.  A forward is 88
+    # dependent kernels, so this times 88 is the part of ms_per_step no kernel can win back.
+    if not args.eager:
+        node_ms = drv.homTimeEmptyGraphNodes(88, 256, 200)
+        if node_ms > 0:
+            kernels["graph_of_88_empty_kernels"] = {
+                "us_per_node": node_ms * 1e3, "us_per_graph": node_ms * 88e3,
+                "note": "floor under the 88 dependent kernel nodes of the b8 x s128 forward"}
+
     # the reference's whole BertForMaskedLM graph: encoder + LM head to logits [8, 128, 30522]
     enc = bert.BertEncoder(d["layers"], d["hidden"], d["heads"], d["ffn"], d["bs"], d["seq"], d["vocab"],
                            gemm_mode=args.gemm_mode, gelu_form="erf", lm_head=True)

@@ -839,6 +839,21 @@ DRV_EXPORT double homMfmaCeilingProbe(int randomOperands, int valuPerMfma) {
   return tflops;
 }
 
+// What one kernel node of a replayed graph costs when the kernel does nothing:
+// `nodes` empty kernels of `groups` workgroups captured into one graph, ms per
+// node over `replays` replays.  The floor under every kernel of the encoder's
+// 88-launch chain.  Negative on error.
+namespace {
+__global__ void emptyNodeKernel() {}
+} // namespace
+DRV_EXPORT double homTimeEmptyGraphNodes(int nodes, int groups, int replays) {
+  if (nodes < 1 || groups < 1 || replays < 1)
+    return -1.0;
+  Timer t;
+  return t.runGraph([&] { emptyNodeKernel<<<groups, 256, 0, t.s>>>(); }, nodes,
+                    replays, 5);
+}
+
 // D = act(A.B + bias) with bias broadcast as a [1,1,N] C (useBias) or beta = 0.
 // gemmNum is 1-based (0 = library picks); returns ms per call.  inGraph != 0:
 // 100 calls per captured graph, iters / 100 replays.

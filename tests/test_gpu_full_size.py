@@ -182,3 +182,7 @@ def test_driver_measurement_helpers(gpu, rt):
     t_zero = drv.homTimeGemmZeroOperands(ROWS, 1024, 4096, 0, 0, idx.value + 1, sk.value, 10, 3)
     assert 0.03 < t_zero < 1.0 and 0.03 < t_rnd < 1.0, (t_zero, t_rnd)
     assert t_zero <= 1.1 * t_rnd, (t_zero, t_rnd)
+    # a node of a replayed graph of empty kernels: a microsecond or two, never zero
+    node_ms = drv.homTimeEmptyGraphNodes(88, 256, 50)
+    assert 2e-4 < node_ms < 2e-2, node_ms
+    assert drv.homTimeEmptyGraphNodes(0, 256, 50) < 0
