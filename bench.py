@@ -319,7 +319,8 @@ def main():
 
     # What the chain of launches itself costs: 88 empty kernels as the nodes of one replayed graph.  A forward is 88
     # dependent kernels, so this times 88 is the part of ms_per_step no kernel can win back.
-    if not args.eager:
+    # (left out under a tracer: its ~20 000 empty dispatches would only pad the trace)
+    if not args.eager and not traced:
         node_ms = drv.homTimeEmptyGraphNodes(88, 256, 200)
         if node_ms > 0:
             kernels["graph_of_88_empty_kernels"] = {
